@@ -1,0 +1,345 @@
+// Routed experts and other products in which every row has a weight matrix of its own choosing.
+//
+//   route_top        per token: the `top` largest of its router logits (the lower index wins a tie) and the softmax
+//                    over those alone, float32.
+//   group_by_expert  the step's (token, choice) pairs grouped by expert, each group padded to whole tiles of 16
+//                    rows: row_token[row] (-1 in the padding), pair_row[pair], tile_expert[tile] (-1 beyond the
+//                    last tile).  One block; no count leaves the device.  The order of a group's rows is whatever
+//                    the block's atomic counters give: a row's result does not depend on its place.
+//   grouped product  out[row] = W[e(row)] a[row] on the matrix cores, e from tile_expert (16 rows a tile share it)
+//                    or, for a batch of independent products (one weight per head, say), from the block's z.
+//                    bfloat16 operands on v_mfma_f32_16x16x32_bf16, float32 operands on v_mfma_f32_16x16x4_f32
+//                    (exact products); float32 sums in the order of k either way, whatever else is in the step.
+//                    With two weights the epilogue forms silu(W0 a) * (W1 a).
+//   combine          out[t] = sum_k weight[t][k] * rows[pair_row[t][k]] in the order of k, float32.
+//
+// Matrix-core layout as in the other products of this package: operand A = the weight tile (lane 16 j + r: row
+// n0 + r, 8 values of k from 32 s + 8 j), operand B = the rows (lane 16 j + r: row r, the same k), result lane
+// 16 j + r holds out[r][n0 + 4 j + i], i = 0..3.
+#include "common.h"
+
+CWM_DEFINE_ERROR_API
+
+#define ROUTE_MAX_TOP 16
+#define ROUTE_MAX_EXPERTS 256
+#define TILE_ROWS 16
+
+extern "C" int cwm_route_max_top() { return ROUTE_MAX_TOP; }
+extern "C" int cwm_route_max_experts() { return ROUTE_MAX_EXPERTS; }
+extern "C" int cwm_route_tile_rows() { return TILE_ROWS; }
+
+__global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ chosen,
+                                                        float* __restrict__ weights, int n_tokens, int n_experts, int top) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tokens) return;
+  const float* z = logits + (size_t)t * n_experts;
+  int idx[ROUTE_MAX_TOP];
+  float val[ROUTE_MAX_TOP];
+#pragma unroll
+  for (int k = 0; k < ROUTE_MAX_TOP; ++k) {
+    idx[k] = -1;
+    val[k] = 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < ROUTE_MAX_TOP; ++k) {
+    if (k < top) {
+      int best = -1;
+      float bv = 0.f;
+      for (int e = 0; e < n_experts; ++e) {
+        bool taken = false;
+#pragma unroll
+        for (int m = 0; m < ROUTE_MAX_TOP; ++m) taken |= (m < k && idx[m] == e);
+        const float v = z[e];
+        if (!taken && (best < 0 || v > bv)) {
+          best = e;
+          bv = v;
+        }
+      }
+      idx[k] = best;
+      val[k] = bv;
+    }
+  }
+  float sum = 0.f;
+  const float largest = val[0];  // the first chosen is the largest
+#pragma unroll
+  for (int k = 0; k < ROUTE_MAX_TOP; ++k)
+    if (k < top) {
+      val[k] = expf(val[k] - largest);
+      sum += val[k];
+    }
+#pragma unroll
+  for (int k = 0; k < ROUTE_MAX_TOP; ++k)
+    if (k < top) {
+      chosen[(size_t)t * top + k] = idx[k];
+      weights[(size_t)t * top + k] = val[k] / sum;
+    }
+}
+
+extern "C" int cwm_route_top(const float* logits, int* chosen, float* weights, int n_tokens, int n_experts, int top,
+                             hipStream_t stream) {
+  CWM_REQUIRE(logits && chosen && weights, "route_top: arguments missing");
+  CWM_REQUIRE(top >= 1 && top <= ROUTE_MAX_TOP && top <= n_experts, "route_top: %d of %d experts, the kernel takes up to %d", top, n_experts,
+              ROUTE_MAX_TOP);
+  if (n_tokens <= 0) return 0;
+  hipLaunchKernelGGL(route_top_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, stream, logits, chosen, weights, n_tokens, n_experts, top);
+  return cwm_launch_status("route_top");
+}
+
+__global__ void __launch_bounds__(1024) group_by_expert_kernel(const int* __restrict__ chosen, int n_pairs, int n_experts,
+                                                               int* __restrict__ row_token, int* __restrict__ pair_row,
+                                                               int* __restrict__ tile_expert, int n_tiles, int top, int tile_align) {
+  __shared__ int count[ROUTE_MAX_EXPERTS];
+  __shared__ int start[ROUTE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
+  for (int i = threadIdx.x; i < n_tiles * TILE_ROWS; i += blockDim.x) row_token[i] = -1;
+  for (int i = threadIdx.x; i < n_tiles; i += blockDim.x) tile_expert[i] = -1;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
+    const int e = chosen[i];
+    if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tile = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      start[e] = tile * TILE_ROWS;
+      const int tiles = (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+      for (int k = 0; k < tiles && tile + k < n_tiles; ++k) tile_expert[tile + k] = e;
+      tile += (tiles + tile_align - 1) / tile_align * tile_align;  // an expert's tiles start at a multiple of tile_align
+      count[e] = 0;
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
+    const int e = chosen[i];
+    int row = -1;
+    if (e >= 0 && e < n_experts) {
+      row = start[e] + atomicAdd(&count[e], 1);
+      if (row < n_tiles * TILE_ROWS)
+        row_token[row] = i / top;
+      else
+        row = -1;
+    }
+    pair_row[i] = row;
+  }
+}
+
+// tile_align: an expert's first tile lies at a multiple of so many tiles (the tiles that one block of the product takes).
+extern "C" int cwm_group_by_expert(const int* chosen, int n_tokens, int top, int n_experts, int* row_token, int* pair_row,
+                                   int* tile_expert, int n_tiles, int tile_align, hipStream_t stream) {
+  CWM_REQUIRE(chosen && row_token && pair_row && tile_expert, "group_by_expert: arguments missing");
+  CWM_REQUIRE(n_experts >= 1 && n_experts <= ROUTE_MAX_EXPERTS && top >= 1, "group_by_expert: %d experts, the kernel takes up to %d", n_experts,
+              ROUTE_MAX_EXPERTS);
+  const long n_pairs = (long)n_tokens * top;
+  CWM_REQUIRE(tile_align >= 1 && (long)n_tiles >= (n_pairs + TILE_ROWS - 1) / TILE_ROWS + (long)n_experts * tile_align,
+              "group_by_expert: %d tiles do not hold %ld pairs of %d experts", n_tiles, n_pairs, n_experts);
+  if (n_tokens <= 0) return 0;
+  hipLaunchKernelGGL(group_by_expert_kernel, dim3(1), dim3(1024), 0, stream, chosen, (int)n_pairs, n_experts, row_token, pair_row, tile_expert,
+                     n_tiles, top, tile_align);
+  return cwm_launch_status("group_by_expert");
+}
+
+// ---- the grouped product ------------------------------------------------------------------------------------- //
+template <typename T> struct Frag;
+template <> struct Frag<bf16_t> {
+  static constexpr int K_STEP = 32;  // values of k one matrix instruction takes
+  static constexpr int PER_LANE = 8;
+  Frag8 f;
+  __device__ __forceinline__ void zero() { f.u = make_uint4(0, 0, 0, 0); }
+  __device__ __forceinline__ void load16(const bf16_t* p) { f.u = *(const uint4*)p; }
+  __device__ __forceinline__ void load_some(const bf16_t* p, int n) {
+    zero();
+    for (int i = 0; i < PER_LANE; ++i)
+      if (i < n) f.h[i] = p[i];
+  }
+  static __device__ __forceinline__ float4v mma(const Frag& w, const Frag& a, float4v acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.f.v, a.f.v, acc, 0, 0, 0);
+  }
+};
+template <> struct Frag<float> {
+  static constexpr int K_STEP = 16;  // four instructions of 4: lane group j supplies k = 4 j + e to instruction e
+  static constexpr int PER_LANE = 4;
+  float4 f;
+  __device__ __forceinline__ void zero() { f = make_float4(0.f, 0.f, 0.f, 0.f); }
+  __device__ __forceinline__ void load16(const float* p) { f = *(const float4*)p; }
+  __device__ __forceinline__ void load_some(const float* p, int n) {
+    f.x = n > 0 ? p[0] : 0.f;
+    f.y = n > 1 ? p[1] : 0.f;
+    f.z = n > 2 ? p[2] : 0.f;
+    f.w = n > 3 ? p[3] : 0.f;
+  }
+  static __device__ __forceinline__ float4v mma(const Frag& w, const Frag& a, float4v acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.f.x, a.f.x, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.f.y, a.f.y, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.f.z, a.f.z, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.f.w, a.f.w, acc, 0, 0, 0);
+    return acc;
+  }
+};
+
+// A block of four wavefronts takes RT row tiles of one expert (they follow one another in the list) and 64 columns;
+// wavefront w the columns 16 w .. 16 w + 15 for all of the block's rows, so a weight tile is loaded once for RT
+// tiles of rows.  VEC: rows of a and W start at multiples of 16 bytes and K is a multiple of a lane's piece.
+template <typename T, int RT, bool GATED, bool VEC>
+__global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
+                                                              const T* __restrict__ w0, const T* __restrict__ w1, long w_stride,
+                                                              const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
+                                                              int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int tile0 = blockIdx.x * RT;
+  int expert;
+  if (tile_expert) {
+    expert = tile0 < n_tiles ? tile_expert[tile0] : -1;
+    if (expert < 0) return;
+  } else {
+    expert = blockIdx.z;
+  }
+  const int n0 = blockIdx.y * 64 + wave * 16;
+  if (n0 >= N) return;
+  const int col = n0 + r;
+  const T* wrow0 = w0 + (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K;
+  const T* wrow1 = GATED ? w1 + (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K : nullptr;
+  const T* arow[RT];
+  bool tile_live[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int tile = tile0 + rt;
+    // a tile of another expert, or beyond the rows, is left out (its rows belong to another block)
+    tile_live[rt] = tile_expert ? (tile < n_tiles && tile_expert[tile] == expert) : tile * TILE_ROWS < n_rows;
+    const int row = tile * TILE_ROWS + r;
+    long src = -1;
+    if (tile_live[rt]) src = row_token ? row_token[row] : (row < n_rows ? row : -1);
+    arow[rt] = src >= 0 ? a + (size_t)blockIdx.z * a_batch + (size_t)src * a_ld : nullptr;
+  }
+  float4v acc0[RT], acc1[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) acc0[rt] = acc1[rt] = (float4v){0.f, 0.f, 0.f, 0.f};
+  constexpr int STEP = Frag<T>::K_STEP, PIECE = Frag<T>::PER_LANE;
+  for (int k0 = 0; k0 < K; k0 += STEP) {
+    const int k = k0 + j * PIECE;
+    const int left = K - k;  // values of this lane's piece inside K
+    Frag<T> fw0, fw1, fa[RT];
+    if (VEC) {
+      if (left > 0) {
+        fw0.load16(wrow0 + k);
+        if (GATED) fw1.load16(wrow1 + k);
+      } else {
+        fw0.zero();
+        if (GATED) fw1.zero();
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (arow[rt] && left > 0)
+          fa[rt].load16(arow[rt] + k);
+        else
+          fa[rt].zero();
+      }
+    } else {
+      fw0.load_some(wrow0 + k, left);
+      if (GATED) fw1.load_some(wrow1 + k, left);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (arow[rt])
+          fa[rt].load_some(arow[rt] + k, left);
+        else
+          fa[rt].zero();
+      }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      acc0[rt] = Frag<T>::mma(fw0, fa[rt], acc0[rt]);
+      if (GATED) acc1[rt] = Frag<T>::mma(fw1, fa[rt], acc1[rt]);
+    }
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if (!tile_live[rt]) continue;
+    const int row = (tile0 + rt) * TILE_ROWS + r;
+    if (!tile_expert && row >= n_rows) continue;
+    const size_t base = (size_t)blockIdx.z * out_batch + (size_t)row * out_ld;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = n0 + 4 * j + i;
+      if (c >= N) continue;
+      float v = acc0[rt][i];
+      if (GATED) v = v / (1.f + expf(-v)) * acc1[rt][i];
+      if (out_dtype == CWM_F32)
+        ((float*)out)[base + c] = v;
+      else
+        ((bf16_t*)out)[base + c] = f32_to_bf16(v);
+    }
+  }
+}
+
+template <typename T, int RT, bool GATED>
+static void launch_grouped(bool vec, dim3 grid, hipStream_t stream, const T* a, long a_ld, long a_batch, const int* row_token, const T* w0,
+                           const T* w1, long w_stride, const int* tile_expert, int n_tiles, void* out, int out_dtype, long out_ld,
+                           long out_batch, int n_rows, int N, int K) {
+  if (vec)
+    hipLaunchKernelGGL((grouped_product_kernel<T, RT, GATED, true>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1, w_stride,
+                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+  else
+    hipLaunchKernelGGL((grouped_product_kernel<T, RT, GATED, false>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1, w_stride,
+                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+}
+
+// a: rows of K values, `a_ld` apart (row `row_token[row]` for list row `row` if a list is given; batch z starts
+// `a_batch` further).  w0 (and w1 for the gated form): [experts or batches][N][K], `w_stride` apart.  With
+// `tile_expert` the rows are the list's n_tiles * 16 and out is [rows][out_ld]; without, every batch z < n_batch
+// multiplies the same n_rows rows by its own weight into out + z * out_batch.
+extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int dtype, const int* row_token, const void* w0, const void* w1,
+                                   long w_stride, const int* tile_expert, int n_tiles, int n_batch, void* out, int out_dtype, long out_ld,
+                                   long out_batch, int n_rows, int N, int K, int tiles_a_block, hipStream_t stream) {
+  CWM_REQUIRE(a && w0 && out, "grouped_product: arguments missing");
+  CWM_REQUIRE(N > 0 && K > 0 && a_ld >= K && out_ld >= 0, "grouped_product: bad sizes");
+  CWM_REQUIRE(tile_expert ? (n_tiles >= 0 && n_batch == 1 && row_token) : (n_batch >= 1 && n_batch <= 65535), "grouped_product: give a tile list or a number of batches");
+  const int tiles = tile_expert ? n_tiles : (n_rows + TILE_ROWS - 1) / TILE_ROWS;
+  if (tiles <= 0) return 0;
+  const int esize = dtype == CWM_BF16 ? 2 : 4;
+  const int piece = dtype == CWM_BF16 ? 8 : 4;
+  const bool vec = K % piece == 0 && (a_ld * esize) % 16 == 0 && (a_batch * esize) % 16 == 0 && (w_stride * esize) % 16 == 0 &&
+                   ((uintptr_t)a % 16) == 0 && ((uintptr_t)w0 % 16) == 0 && (!w1 || ((uintptr_t)w1 % 16) == 0);
+  // many rows an expert: four row tiles share each weight tile; few: one, so that more blocks stream the weights
+  CWM_REQUIRE(tiles_a_block == 1 || tiles_a_block == 4, "grouped_product: a block takes 1 or 4 row tiles");
+  const bool wide = tiles_a_block == 4;
+  const int rt = tiles_a_block;
+  dim3 grid((tiles + rt - 1) / rt, (N + 63) / 64, tile_expert ? 1 : n_batch);
+  CWM_REQUIRE(grid.y <= 65535, "grouped_product: too many columns");
+#define CWM_GROUPED(T, RT, GATED)                                                                                                      \
+  launch_grouped<T, RT, GATED>(vec, grid, stream, (const T*)a, a_ld, a_batch, row_token, (const T*)w0, (const T*)w1, w_stride, tile_expert, \
+                               n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K)
+  if (dtype == CWM_BF16) {
+    if (w1) { if (wide) CWM_GROUPED(bf16_t, 4, true); else CWM_GROUPED(bf16_t, 1, true); }
+    else    { if (wide) CWM_GROUPED(bf16_t, 4, false); else CWM_GROUPED(bf16_t, 1, false); }
+  } else if (dtype == CWM_F32) {
+    if (w1) { if (wide) CWM_GROUPED(float, 4, true); else CWM_GROUPED(float, 1, true); }
+    else    { if (wide) CWM_GROUPED(float, 4, false); else CWM_GROUPED(float, 1, false); }
+  } else {
+    return cwm_fail("grouped_product: unknown dtype %d", dtype);
+  }
+#undef CWM_GROUPED
+  return cwm_launch_status("grouped_product");
+}
+
+__global__ void __launch_bounds__(256) combine_routed_kernel(const float* __restrict__ rows, long rows_ld, const int* __restrict__ pair_row,
+                                                             const float* __restrict__ weights, float* __restrict__ out, int top, int dim) {
+  const size_t t = blockIdx.x;
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < dim; i += gridDim.y * blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int row = pair_row[t * top + k];
+      if (row >= 0) acc += weights[t * top + k] * rows[(size_t)row * rows_ld + i];
+    }
+    out[t * dim + i] = acc;
+  }
+}
+
+extern "C" int cwm_combine_routed(const float* rows, long rows_ld, const int* pair_row, const float* weights, float* out, int n_tokens,
+                                  int top, int dim, hipStream_t stream) {
+  CWM_REQUIRE(rows && pair_row && weights && out && top >= 1 && dim > 0, "combine_routed: bad arguments");
+  if (n_tokens <= 0) return 0;
+  hipLaunchKernelGGL(combine_routed_kernel, dim3(n_tokens, (dim + 1023) / 1024), dim3(256), 0, stream, rows, rows_ld, pair_row, weights, out, top, dim);
+  return cwm_launch_status("combine_routed");
+}

@@ -1,4 +1,4 @@
 from .model import Model
-from . import llama3_dense  # noqa: F401  (registers the architecture)
+from . import llama3_dense, lapevik  # noqa: F401  (register the architectures)
 
 __all__ = ["Model"]

@@ -1196,3 +1196,14 @@ def measure_mfma_rate(device: torch.device, blocks: int, rounds: int, launches: 
             torch.cuda.synchronize(device)
     flops = lib.cwm_ceiling_mfma_flops(ctypes.c_int(blocks), ctypes.c_int(rounds)) * launches
     return flops / (start.elapsed_time(end) * 1e-3) / 1e15
+
+
+# --------------------------------------------------------------------------- #
+# entry points that live in modules of their own; parts reach them as `ops.<name>` like the ones above
+from .sequence import (  # noqa: E402
+    MAX_CONV_TAPS, MAX_SSM_STATE, add_rows, cast_rows, causal_conv_silu, group_rmsnorm, selective_scan, sigmoid_mul, token_shift,
+)
+from .routed import (  # noqa: E402
+    MAX_EXPERTS, MAX_ROUTE_TOP, ExpertGroups, absorb_queries, combine_routed, expand_values, group_by_expert, grouped_gate_up,
+    grouped_linear, route_top,
+)

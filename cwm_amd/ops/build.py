@@ -55,6 +55,9 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "gemm_bf16_stream": ({},),
     "gemm_bf16_tile": ({},),
     "ceilings": ({},),
+    "groupnorm": ({},),
+    "state_space": ({},),
+    "routed": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),
 }
 

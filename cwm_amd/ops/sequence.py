@@ -1,0 +1,231 @@
+"""Entry points of the row-wise and sequential kernels of layers with group norms, token shift, a selective
+state space and gates (`csrc/groupnorm.hip`, `csrc/state_space.hip`).  Shapes, types and devices are checked on
+the host; there is no CPU path."""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Any, Optional
+
+import torch
+
+from . import build as _build
+
+MAX_CONV_TAPS = 8  # csrc/state_space.hip: CONV_MAX_TAPS
+MAX_SSM_STATE = 256  # csrc/state_space.hip: SCAN_ROWS * 16
+
+
+def _base():
+    from . import KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream  # the shared helpers of this package
+
+    return KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream
+
+
+def _rows_2d(t: torch.Tensor, what: str) -> None:
+    KernelError = _base()[0]
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{what} must be [rows, n] with contiguous rows, found {tuple(t.shape)} with strides {t.stride()}")
+
+
+def group_rmsnorm(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    groups: int,
+    eps: float,
+    out_dtype: torch.dtype,
+    rows: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    accumulate: bool = False,
+    gate: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """weight * x_g / sqrt(mean(x_g^2) + eps) for each of `groups` equal consecutive parts x_g of every row, float32
+    arithmetic.  `x` is [T, D] (rows may lie apart) or float32 partial sums [P, T, D], added in order first; with
+    `gate` ([T, D]) the row is multiplied by silu(gate) before the norm.  `rows` (int32 [R]) chooses rows.  The
+    result goes to a new [R, D] tensor of `out_dtype`, or into `out` ([R, D], which may be `x` itself), added to what
+    is there if `accumulate`."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(x, weight, rows, out, gate)
+    n_partials, partial_stride = 1, 0
+    if x.dim() == 3:
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelError("partial sums must be a contiguous float32 [P, T, D] tensor")
+        n_partials, partial_stride = x.shape[0], x.shape[1] * x.shape[2]
+        n_tokens, dim, src_ld = x.shape[1], x.shape[2], x.shape[2]
+    else:
+        _rows_2d(x, "x")
+        n_tokens, dim = x.shape
+        src_ld = x.stride(0) if n_tokens > 1 else dim
+    if weight.shape != (dim,) or not weight.is_contiguous():
+        raise KernelError(f"norm weight has shape {tuple(weight.shape)}, expected ({dim},)")
+    if groups < 1 or dim % groups != 0:
+        raise KernelError(f"{dim} elements do not divide into {groups} groups")
+    if rows is not None:
+        _i32(rows, "rows")
+    n_out = n_tokens if rows is None else rows.numel()
+    if out is None:
+        if accumulate:
+            raise KernelError("accumulate needs a tensor to add into")
+        out = torch.empty((n_out, dim), dtype=out_dtype, device=x.device)
+    else:
+        _rows_2d(out, "out")
+        if tuple(out.shape) != (n_out, dim):
+            raise KernelError(f"out {tuple(out.shape)} does not fit {n_out} rows of {dim}")
+    gate_ld = 0
+    if gate is not None:
+        _rows_2d(gate, "gate")
+        if tuple(gate.shape) != (n_tokens, dim):
+            raise KernelError(f"gate {tuple(gate.shape)} does not fit x")
+        gate_ld = gate.stride(0) if n_tokens > 1 else dim
+    lib = _build.load("groupnorm")
+    _check(
+        lib,
+        lib.cwm_group_norm(
+            _ptr(x), ctypes.c_int(_code(x.dtype)), ctypes.c_long(src_ld), ctypes.c_int(n_partials), ctypes.c_long(partial_stride),
+            _ptr(gate), ctypes.c_int(_code(gate.dtype) if gate is not None else 0), ctypes.c_long(gate_ld),
+            _ptr(weight), ctypes.c_int(_code(weight.dtype)), _ptr(out), ctypes.c_int(_code(out.dtype)),
+            ctypes.c_long(out.stride(0) if n_out > 1 else dim), _ptr(rows), ctypes.c_int(n_out), ctypes.c_int(dim), ctypes.c_int(groups),
+            ctypes.c_float(eps), ctypes.c_int(int(accumulate)), _stream(),
+        ),
+    )
+    return out
+
+
+def add_rows(h: torch.Tensor, delta: torch.Tensor) -> None:
+    """h (float32 [T, D]) += delta ([T, D], or partial sums [P, T, D] added in order)."""
+    if delta.dim() == 3:
+        for p in range(delta.shape[0]):
+            h.add_(delta[p])
+    else:
+        h.add_(delta)
+
+
+def cast_rows(h: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 rows in `dtype` (the rows themselves if that is float32)."""
+    if h.dtype == dtype:
+        return h
+    from . import sum_partials
+
+    return sum_partials(h.unsqueeze(0), dtype)
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, batch: Any, out_dtype: torch.dtype, write_state: bool = True) -> torch.Tensor:
+    """s_t = h_t + (h_(t-1) - h_t) * mu for the step's tokens: `h` float32 [T, D]; the row before a portion's first
+    token is the sequence's row of `state` (float32 [slots, D]; zero at position 0), which then receives the
+    portion's last row."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(h, mu, state)
+    if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+        raise KernelError("the stream must be a contiguous float32 [T, D] tensor")
+    n_tokens, dim = h.shape
+    if mu.dtype != torch.float32 or mu.shape != (dim,) or not mu.is_contiguous():
+        raise KernelError(f"mu must be float32 [{dim}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != dim or not state.is_contiguous():
+        raise KernelError(f"the state must be float32 [slots, {dim}]")
+    if n_tokens != batch.n_tokens:
+        raise KernelError("one row per token of the step is needed")
+    out = torch.empty((n_tokens, dim), dtype=out_dtype, device=h.device)
+    lib = _build.load("groupnorm")
+    _check(
+        lib,
+        lib.cwm_token_shift(
+            _ptr(h), _ptr(mu), _ptr(state), _ptr(batch.state_slots), _ptr(batch.cu_q), _ptr(batch.seq_of_token), _ptr(batch.positions),
+            _ptr(out), ctypes.c_int(_code(out_dtype)), ctypes.c_int(n_tokens), ctypes.c_int(dim), ctypes.c_int(state.shape[0]),
+            ctypes.c_int(int(write_state)), _stream(),
+        ),
+    )
+    return out
+
+
+def sigmoid_mul(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """a * sigmoid(gate), both [T, n] of one type (rows may lie apart); float32 arithmetic."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(a, gate)
+    _rows_2d(a, "a")
+    _rows_2d(gate, "gate")
+    if a.shape != gate.shape or a.dtype != gate.dtype:
+        raise KernelError(f"a {tuple(a.shape)} {a.dtype} and gate {tuple(gate.shape)} {gate.dtype} do not match")
+    n, width = a.shape
+    out = torch.empty((n, width), dtype=a.dtype, device=a.device)
+    lib = _build.load("groupnorm")
+    _check(
+        lib,
+        lib.cwm_sigmoid_mul(
+            _ptr(a), ctypes.c_long(a.stride(0) if n > 1 else width), _ptr(gate), ctypes.c_long(gate.stride(0) if n > 1 else width),
+            _ptr(out), ctypes.c_long(width), ctypes.c_int(_code(a.dtype)), ctypes.c_int(n), ctypes.c_int(width), _stream(),
+        ),
+    )
+    return out
+
+
+def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, state_offset: int, batch: Any) -> torch.Tensor:
+    """silu(bias + causal convolution) per channel over each sequence of the step: `x` [T, C] (rows may lie apart),
+    `weight` float32 [C, taps] (the last column is the current token's), `bias` float32 [C].  A sequence's last
+    taps - 1 inputs live in its row of `state` (float32 [slots, n]) from `state_offset` on, [taps - 1, C] oldest
+    first: read by the portion's first tokens, then replaced.  Returns [T, C] in the type of `x`."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(x, weight, bias, state)
+    _rows_2d(x, "x")
+    n_tokens, channels = x.shape
+    if weight.dtype != torch.float32 or weight.dim() != 2 or weight.shape[0] != channels or not weight.is_contiguous():
+        raise KernelError(f"the convolution's weight must be float32 [{channels}, taps]")
+    taps = weight.shape[1]
+    if bias.dtype != torch.float32 or bias.shape != (channels,) or not bias.is_contiguous():
+        raise KernelError(f"the convolution's bias must be float32 [{channels}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous():
+        raise KernelError("the state must be a contiguous float32 [slots, n] tensor")
+    if state_offset < 0 or state_offset + (taps - 1) * channels > state.shape[1]:
+        raise KernelError("the state row does not hold the convolution's inputs")
+    if n_tokens != batch.n_tokens:
+        raise KernelError("one row per token of the step is needed")
+    out = torch.empty((n_tokens, channels), dtype=x.dtype, device=x.device)
+    lib = _build.load("state_space")
+    _check(
+        lib,
+        lib.cwm_conv_silu(
+            _ptr(x), ctypes.c_long(x.stride(0) if n_tokens > 1 else channels), ctypes.c_int(_code(x.dtype)), _ptr(weight), _ptr(bias),
+            _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_long(state_offset), _ptr(batch.state_slots), _ptr(batch.cu_q),
+            _ptr(batch.seq_of_token), _ptr(out), ctypes.c_int(n_tokens), ctypes.c_int(channels), ctypes.c_int(taps),
+            ctypes.c_int(state.shape[0]), _stream(),
+        ),
+    )
+    return out
+
+
+def selective_scan(
+    xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, batch: Any,
+    heads: int, head_dim: int, n_state: int, groups: int,
+) -> torch.Tensor:
+    """The recurrence S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x per head over each sequence of the step,
+    in float32, from and into the sequences' rows of `state` (float32 [slots, n], S of all heads first, each
+    [n_state, head_dim]).  `xbc` [T, heads * head_dim + 2 * groups * n_state] = [x | B | C]; `dt` [T, heads] before
+    bias and softplus (rows may lie apart); `dt_bias`, `a_log`, `d_skip` float32 [heads].  Returns y float32
+    [T, heads * head_dim]."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(xbc, dt, dt_bias, a_log, d_skip, state)
+    _rows_2d(xbc, "xbc")
+    _rows_2d(dt, "dt")
+    n_tokens = xbc.shape[0]
+    inner = heads * head_dim
+    if xbc.shape[1] != inner + 2 * groups * n_state or dt.shape != (n_tokens, heads) or dt.dtype != xbc.dtype:
+        raise KernelError(f"xbc {tuple(xbc.shape)} and dt {tuple(dt.shape)} do not fit {heads} heads of {head_dim} with {groups} groups of {n_state}")
+    for name, t in (("dt_bias", dt_bias), ("A_log", a_log), ("D", d_skip)):
+        if t.dtype != torch.float32 or t.shape != (heads,) or not t.is_contiguous():
+            raise KernelError(f"{name} must be float32 [{heads}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or state.shape[1] < heads * n_state * head_dim:
+        raise KernelError("the state must be a contiguous float32 [slots, n] tensor that holds every head's state")
+    if n_state > MAX_SSM_STATE:
+        raise KernelError(f"a state of {n_state} rows is more than the {MAX_SSM_STATE} the scan kernel takes")
+    if n_tokens != batch.n_tokens:
+        raise KernelError("one row per token of the step is needed")
+    y = torch.empty((n_tokens, inner), dtype=torch.float32, device=xbc.device)
+    lib = _build.load("state_space")
+    _check(
+        lib,
+        lib.cwm_selective_scan(
+            _ptr(xbc), ctypes.c_long(xbc.stride(0) if n_tokens > 1 else xbc.shape[1]), _ptr(dt), ctypes.c_long(dt.stride(0) if n_tokens > 1 else heads),
+            ctypes.c_int(_code(xbc.dtype)), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state), ctypes.c_long(state.shape[1]),
+            _ptr(batch.state_slots), _ptr(batch.cu_q), _ptr(y), ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs), ctypes.c_int(heads),
+            ctypes.c_int(head_dim), ctypes.c_int(n_state), ctypes.c_int(groups), ctypes.c_int(state.shape[0]), _stream(),
+        ),
+    )
+    return y

@@ -26,11 +26,15 @@ from .base import (
     TensorSpec,
     register_part,
 )
-from . import norm, rope, attention, feedforward, block, embedding  # noqa: F401  (fill the registries)
+from . import norm, rope, attention, feedforward, block, embedding, token_shift, state_space, latent_attention, experts  # noqa: F401  (fill the registries)
 from .linear import LinearWeights
-from .norm import RMSNorm
+from .norm import GroupRMSNorm, RMSNorm
 from .rope import NoPositionEncoding, RotaryEncoding, llama3_scale_frequencies, rotary_inverse_frequencies
 from .attention import PagedAttention
 from .feedforward import SwiGLU
-from .block import PreNormBlock
-from .embedding import LinearHead, TokenEmbedding
+from .block import PostNormBlock, PreNormBlock
+from .embedding import LinearHead, NormedTokenEmbedding, TokenEmbedding
+from .token_shift import TokenShift
+from .state_space import SelectiveStateSpace
+from .latent_attention import LatentAttention
+from .experts import RoutedExperts

@@ -31,3 +31,46 @@ class PreNormBlock(Block):
 
 
 register_part("block", "pre_norm", PreNormBlock)
+
+
+class PostNormBlock(Block):
+    """h += norm1(mixer(s)); h += norm2(feed_forward(h)): each sublayer reads the residual stream itself and its
+    output is normalised before it joins the stream.  What the mixer reads, s, is the stream after the block's
+    `shift` (a mixer of its own with its own state, a token shift for instance), or the stream itself in the
+    activation type where the layer has none.  A layer without a feed-forward names neither `feed_forward`
+    nor `norm2`.  The norms add into the stream themselves (`add_normed`), so the block leaves no pending update."""
+
+    def __init__(
+        self, names: Mapping[str, str], mixer: Mixer, norm1: Norm, shift: Optional[Mixer] = None,
+        feed_forward: Optional[FeedForward] = None, norm2: Optional[Norm] = None,
+    ) -> None:
+        if (feed_forward is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
+        parts = {}
+        if shift is not None:
+            parts["shift"] = shift
+        parts.update(mixer=mixer, norm1=norm1)
+        if feed_forward is not None:
+            parts.update(feed_forward=feed_forward, norm2=norm2)
+        super().__init__(names, **parts)
+        self.shift, self.mixer, self.norm1, self.feed_forward, self.norm2 = shift, mixer, norm1, feed_forward, norm2
+
+    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], batch: Any, cache: Any, write_cache: bool = True) -> None:
+        from .. import ops
+
+        if delta is not None:
+            ops.add_rows(h, delta)
+        act = self.runtime.act_dtype
+        if self.shift is not None:
+            shift_cache, mixer_cache = cache
+            s = self.shift.forward(h, batch, shift_cache, write_cache)
+        else:
+            mixer_cache = cache
+            s = ops.cast_rows(h, act)
+        self.norm1.add_normed(h, self.mixer.forward(s, batch, mixer_cache, write_cache))
+        if self.feed_forward is not None:
+            self.norm2.add_normed(h, self.feed_forward.forward(ops.cast_rows(h, act), batch))
+        return None
+
+
+register_part("block", "post_norm", PostNormBlock)

@@ -7,7 +7,7 @@ from typing import Any, Dict, Mapping, Optional
 import torch
 
 from .. import ops
-from .base import Embedding, Head, Runtime, TensorSpec, register_part
+from .base import Embedding, Head, PartChoice, Runtime, TensorSpec, register_part
 from .linear import LinearWeights
 
 
@@ -17,20 +17,54 @@ class TokenEmbedding(Embedding):
 
     replayable = True
 
-    def __init__(self, vocab_size: int, dim: int, scale: Optional[float] = None) -> None:
+    def __init__(self, vocab_size: int, dim: int, scale: Optional[float] = None, tensor: str = "weight") -> None:
+        """`tensor`: the table's local name ("" where the folder names it by the part's prefix alone)."""
         self.vocab_size = vocab_size
         self.dim = dim
         self.scale = 1.0 if scale is None else float(scale)
+        self.tensor = tensor
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.vocab_size, self.dim))}
+        return {self.tensor: TensorSpec((self.vocab_size, self.dim))}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        self.table = tensors["weight"].contiguous()
+        self.table = tensors[self.tensor].contiguous()
 
     def forward(self, batch: Any) -> torch.Tensor:
         return ops.embedding(batch.tokens, self.table, self.scale)
+
+
+class NormedTokenEmbedding(TokenEmbedding):
+    """The table's rows, normalised: h = norm(scale * table[tokens]).  `norm` is any norm part that can
+    normalise rows where they lie (`normalize_`); its tensors carry `norm_prefix` after the table's name."""
+
+    def __init__(
+        self, vocab_size: int, dim: int, norm: PartChoice, scale: Optional[float] = None, tensor: str = "weight", norm_prefix: str = "norm.",
+    ) -> None:
+        super().__init__(vocab_size, dim, scale, tensor)
+        self.norm = norm.build("norm")
+        self.norm_prefix = norm_prefix
+        if not hasattr(self.norm, "normalize_"):
+            raise TypeError(f"the norm {norm.name!r} cannot normalise rows in place")
+
+    @property
+    def replayable(self) -> bool:  # type: ignore[override]
+        return self.norm.replayable
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = super().tensor_specs()
+        for name, spec in self.norm.tensor_specs().items():
+            specs[self.norm_prefix + name] = spec
+        return specs
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        n = len(self.norm_prefix)
+        self.norm.bind({name[n:]: t for name, t in tensors.items() if name != self.tensor and name.startswith(self.norm_prefix)}, runtime)
+
+    def forward(self, batch: Any) -> torch.Tensor:
+        return self.norm.normalize_(super().forward(batch))
 
 
 class LinearHead(Head):
@@ -39,20 +73,22 @@ class LinearHead(Head):
 
     replayable = True
 
-    def __init__(self, vocab_size: int, dim: int) -> None:
+    def __init__(self, vocab_size: int, dim: int, tensor: str = "weight") -> None:
         self.vocab_size = vocab_size
         self.dim = dim
+        self.tensor = tensor
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.vocab_size, self.dim))}
+        return {self.tensor: TensorSpec((self.vocab_size, self.dim))}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        self.weights = LinearWeights(tensors["weight"], stream_copy=runtime.stream_copies)
+        self.weights = LinearWeights(tensors[self.tensor], stream_copy=runtime.stream_copies)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.weights(x, out_dtype=torch.float32)
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("embedding", "normed_embedding", NormedTokenEmbedding)
 register_part("head", "linear_head", LinearHead)

@@ -34,3 +34,52 @@ class RMSNorm(Norm):
 
 
 register_part("norm", "rmsnorm", RMSNorm)
+
+
+class GroupRMSNorm(Norm):
+    """RMSNorm in `groups` equal consecutive parts: each part of a row is divided by its own
+    sqrt(mean(part^2) + eps), and the whole row is multiplied by the weight; float32 arithmetic.  One group is
+    the plain RMSNorm.  `tensor` is the weight's local name ("" where the folder names the weight by the part's
+    prefix alone).
+
+    Besides the norm-after-sum of `forward` it serves layers that normalise a sublayer's output before the
+    residual sum (`add_normed`) and rows that are normalised where they lie (`normalize_`)."""
+
+    replayable = True
+
+    def __init__(self, dim: int, eps: float, groups: int = 1, tensor: str = "weight") -> None:
+        if groups < 1 or dim % groups != 0:
+            raise ValueError(f"{dim} elements do not divide into {groups} groups")
+        self.dim = dim
+        self.eps = float(eps)
+        self.groups = groups
+        self.tensor = tensor
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.tensor: TensorSpec((self.dim,), init="norm", precision="stored")}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.weight = tensors[self.tensor].contiguous()
+
+    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if delta is not None:
+            if rows is not None:
+                raise ValueError("a pending residual update with a choice of rows is not served by the group norm")
+            ops.add_rows(h, delta)
+        return ops.group_rmsnorm(h, self.weight, self.groups, self.eps, self.runtime.act_dtype, rows=rows)
+
+    def add_normed(self, h: torch.Tensor, y: torch.Tensor) -> None:
+        """h (float32 [T, D]) += norm(y) * weight; `y` is [T, D] or float32 partial sums [P, T, D]."""
+        ops.group_rmsnorm(y, self.weight, self.groups, self.eps, torch.float32, out=h, accumulate=True)
+
+    def normalize_(self, x: torch.Tensor) -> torch.Tensor:
+        """Rows of `x` ([T, D], the rows may lie apart) normalised in place."""
+        return ops.group_rmsnorm(x, self.weight, self.groups, self.eps, x.dtype, out=x)
+
+    def gated(self, y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+        """norm(y * silu(gate)) * weight in the activation type: the gate is applied before the norm."""
+        return ops.group_rmsnorm(y, self.weight, self.groups, self.eps, self.runtime.act_dtype, gate=gate)
+
+
+register_part("norm", "group_rmsnorm", GroupRMSNorm)

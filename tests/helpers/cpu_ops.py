@@ -173,12 +173,131 @@ def token_logprobs(logits, rows, targets):
     return lp.gather(1, targets.long()[:, None])[:, 0]
 
 
+# ---- layers with group norms, token shift, a selective state space, a latent attention and routed experts ---- #
+def group_rmsnorm(x, weight, groups, eps, out_dtype, rows=None, out=None, accumulate=False, gate=None):
+    v = x.float().sum(0) if x.dim() == 3 else x.float()
+    if gate is not None:
+        g = gate.float()
+        v = v * (g * torch.sigmoid(g))
+    if rows is not None:
+        v = v[rows.long()]
+    parts = v.reshape(v.shape[0], groups, -1)
+    parts = parts / torch.sqrt((parts * parts).mean(-1, keepdim=True) + eps)
+    y = parts.reshape(v.shape) * weight.float()
+    if out is None:
+        return y.to(out_dtype)
+    if accumulate:
+        out += y.to(out.dtype)
+    else:
+        out.copy_(y.to(out.dtype))
+    return out
+
+
+def cast_rows(h, dtype):
+    return h if h.dtype == dtype else h.to(dtype)
+
+
+def token_shift(h, mu, state, batch, out_dtype, write_state=True):
+    out = torch.empty(h.shape, dtype=torch.float32)
+    for b in range(batch.n_seqs):
+        lo, hi = int(batch.cu_q[b]), int(batch.cu_q[b + 1])
+        slot = int(batch.state_slots[b])
+        first = torch.zeros_like(h[0]) if int(batch.positions[lo]) == 0 else state[slot].clone()
+        prev = torch.cat([first[None], h[lo : hi - 1]], 0)
+        out[lo:hi] = h[lo:hi] + (prev - h[lo:hi]) * mu
+        if write_state:
+            state[slot] = h[hi - 1]
+    return out.to(out_dtype)
+
+
+def sigmoid_mul(a, gate):
+    return (a.float() * torch.sigmoid(gate.float())).to(a.dtype)
+
+
+def causal_conv_silu(x, weight, bias, state, state_offset, batch):
+    taps, channels = weight.shape[1], x.shape[1]
+    out = torch.empty(x.shape, dtype=torch.float32)
+    for b in range(batch.n_seqs):
+        lo, hi = int(batch.cu_q[b]), int(batch.cu_q[b + 1])
+        slot = int(batch.state_slots[b])
+        kept = state[slot, state_offset : state_offset + (taps - 1) * channels].reshape(taps - 1, channels)
+        seq = torch.cat([kept, x[lo:hi].float()], 0)
+        acc = bias.expand(hi - lo, -1).clone()
+        for k in range(taps):
+            acc = acc + seq[k : k + hi - lo] * weight[:, k]
+        out[lo:hi] = acc * torch.sigmoid(acc)
+        state[slot, state_offset : state_offset + (taps - 1) * channels] = seq[seq.shape[0] - (taps - 1) :].reshape(-1)
+    return out.to(x.dtype)
+
+
+def selective_scan(xbc, dt, dt_bias, a_log, d_skip, state, batch, heads, head_dim, n_state, groups):
+    inner = heads * head_dim
+    y = torch.empty((xbc.shape[0], inner), dtype=torch.float32)
+    per_group = heads // groups
+    for b in range(batch.n_seqs):
+        lo, hi = int(batch.cu_q[b]), int(batch.cu_q[b + 1])
+        slot = int(batch.state_slots[b])
+        carry = state[slot, : heads * n_state * head_dim].reshape(heads, n_state, head_dim).clone()
+        for t in range(lo, hi):
+            row = xbc[t].float()
+            x = row[:inner].reshape(heads, head_dim)
+            bm = row[inner : inner + groups * n_state].reshape(groups, n_state).repeat_interleave(per_group, 0)
+            cm = row[inner + groups * n_state :].reshape(groups, n_state).repeat_interleave(per_group, 0)
+            step = torch.nn.functional.softplus(dt[t].float() + dt_bias)
+            decay = torch.exp(-torch.exp(a_log) * step)
+            carry = decay[:, None, None] * carry + step[:, None, None] * bm[:, :, None] * x[:, None, :]
+            y[t] = (torch.einsum("hnp,hn->hp", carry, cm) + d_skip[:, None] * x).reshape(-1)
+        state[slot, : heads * n_state * head_dim] = carry.reshape(-1)
+    return y
+
+
+def route_top(logits, top):
+    order = torch.sort(logits, dim=-1, descending=True, stable=True)
+    values, chosen = order.values[:, :top], order.indices[:, :top]
+    return chosen.to(torch.int32), torch.softmax(values, -1)
+
+
+def group_by_expert(chosen, n_experts):
+    return chosen  # the stand-ins keep one row a pair, in the order of the pairs
+
+
+def grouped_gate_up(x, groups, gate, up):
+    e = groups.reshape(-1).long()
+    rows = x.float().repeat_interleave(groups.shape[1], 0)
+    g = torch.einsum("rd,rfd->rf", rows, gate.float()[e])
+    u = torch.einsum("rd,rfd->rf", rows, up.float()[e])
+    return (g * torch.sigmoid(g) * u).to(x.dtype)
+
+
+def grouped_linear(rows, groups, weight):
+    return torch.einsum("rf,rdf->rd", rows.float(), weight.float()[groups.reshape(-1).long()])
+
+
+def combine_routed(rows, groups, weights):
+    n, top = weights.shape
+    return (rows.reshape(n, top, -1) * weights[:, :, None]).sum(1)
+
+
+def absorb_queries(q, lead, weight):
+    rest = torch.einsum("thd,hnd->thn", q[:, :, lead:].float(), weight.float())
+    return torch.cat([q[:, :, :lead].float(), rest], -1).to(q.dtype).contiguous()
+
+
+def expand_values(mixed, lead, weight):
+    return torch.einsum("thn,hvn->thv", mixed[:, :, lead:].float(), weight.float()).reshape(mixed.shape[0], -1).to(mixed.dtype)
+
+
+STAND_INS = (
+    "embedding", "add_rmsnorm", "silu_mul", "gate_up_silu", "linear", "gemm_f32", "gemm_bf16",
+    "rope_kv_write", "qkv_rope_write", "paged_attention", "sample", "sample_packed", "token_logprobs",
+    "group_rmsnorm", "cast_rows", "token_shift", "sigmoid_mul", "causal_conv_silu", "selective_scan", "route_top",
+    "group_by_expert", "grouped_gate_up", "grouped_linear", "combine_routed", "absorb_queries", "expand_values",
+)
+
+
 def install(monkeypatch) -> None:
     """Patch every kernel entry point of `cwm_amd.ops` with its stand-in."""
     import cwm_amd.ops as ops
 
-    for name in (
-        "embedding", "add_rmsnorm", "silu_mul", "gate_up_silu", "linear", "gemm_f32", "gemm_bf16",
-        "rope_kv_write", "qkv_rope_write", "paged_attention", "sample", "sample_packed", "token_logprobs",
-    ):
+    for name in STAND_INS:
         monkeypatch.setattr(ops, name, globals()[name])
