@@ -131,11 +131,16 @@ class ShapeBench:
         self.page = page
         self.graphs = graphs
         config = dict(shape)
-        self.full_layers = shape["n_layers"]
-        self.layers = self.full_layers if layers is None else layers
-        config["n_layers"] = self.layers
-        if "window_attn" in shape:
-            config["layer_types"] = layer_kinds(self.layers)
+        if "n_layers" in shape:
+            self.full_layers = shape["n_layers"]
+            self.layers = self.full_layers if layers is None else layers
+            config["n_layers"] = self.layers
+            if "window_attn" in shape:
+                config["layer_types"] = layer_kinds(self.layers)
+        else:  # an architecture that lists its layers
+            self.full_layers = len(shape["layers"])
+            self.layers = self.full_layers if layers is None else layers
+            config["layers"] = list(shape["layers"])[: self.layers]
         t0 = time.time()
         self.model, self.typed = random_model(config, seed=0, dtype=dtype, device=device)
         torch.cuda.synchronize()
@@ -150,6 +155,12 @@ class ShapeBench:
         self.head_params = 0
         head_names = model.tensor_names("head")
         embedding_only = model.tensor_names("embedding") - head_names  # tables of which a step reads one row a token
+        # routed experts: a token is multiplied with `top` of a layer's `n_experts` expert matrices only
+        routed = {}
+        for layer, block in zip(model.plan.layers, model.blocks):
+            for role, part in block.parts.items():
+                if hasattr(part, "n_experts") and hasattr(part, "top"):
+                    routed[layer.prefix + block.names[role] + "e"] = part.top / part.n_experts
         for name, spec in model.tensor_specs().items():
             count = 1
             for n in spec.shape:
@@ -161,11 +172,12 @@ class ShapeBench:
                 if name in head_names:
                     self.head_params += count
                 else:
-                    self.matrix_params += count
+                    share = next((f for prefix, f in routed.items() if name.startswith(prefix)), 1.0)
+                    self.matrix_params += int(count * share)
         self.paged = [spec for spec in model.cache_specs if isinstance(spec, PagedKVSpec)]
         self.windows = sorted({spec.window for spec in self.paged if spec.window is not None})
         self.sampler = Sampler(device)
-        self.vocab = self.typed.vocab_size
+        self.vocab = model.vocab_size
 
     def close(self):
         import gc
@@ -189,13 +201,13 @@ class ShapeBench:
         """Flops of a portion of `n_tokens` after `offset` cached tokens whose last token's logits are wanted:
         2 for every matrix entry and token, the causal attention's two products, and the head for one row."""
         attn = 0
-        for call, slot in zip(self.model.run_order, self.model.cache_slot):
-            spec = self.model.cache_specs[slot] if slot is not None else None
-            if spec in self.paged:
-                # token p reads min(p + 1, window) keys; 2 products (QK^T and PV) of 2 flops, for every query head
-                keys = sum(min(p + 1, spec.window or (p + 1)) for p in range(offset, offset + n_tokens))
-                query_heads = getattr(self.model.blocks[call.layer].mixers()[0], "n_heads", spec.n_kv_heads)
-                attn += 4 * keys * query_heads * spec.head_dim
+        for call, slots in zip(self.model.run_order, self.model.cache_slots):
+            for mixer, slot in zip(self.model.blocks[call.layer].mixers(), slots):
+                spec = self.model.cache_specs[slot]
+                if spec in self.paged:
+                    # token p reads min(p + 1, window) keys; 2 products (QK^T and PV) of 2 flops, for every query head
+                    keys = sum(min(p + 1, spec.window or (p + 1)) for p in range(offset, offset + n_tokens))
+                    attn += 4 * keys * getattr(mixer, "n_heads", spec.n_kv_heads) * spec.head_dim
         return 2 * n_tokens * self.matrix_params + attn + 2 * self.head_params
 
     def make_runner(self, batch, ctx, extra, step_tokens=1):
@@ -283,6 +295,63 @@ class ShapeBench:
         return best
 
 
+def lapevik_config(width, layers, heads, kv_rank, q_rank, ssm_heads, state, groups, ff, experts, top, vocab=32768):
+    """A Lapevik model of `layers` layers, three state-space layers to one latent attention, routed experts in each."""
+    attention = {
+        "type": "latent_attention",
+        "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": kv_rank, "q_rank": q_rank, "scale": 192 ** -0.5,
+                  "rot": {"base": 10000.0, "dims": 64}},
+    }
+    state_space = {"type": "mamba2", "mixer": {"heads": ssm_heads, "vdim": 64, "state": state, "groups": groups, "norm_groups": groups, "conv": 4}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    return {
+        "architecture": "Lapevik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5, "groups": 4},
+        "layers": [dict(attention if i % 4 == 3 else state_space, mlp=mlp) for i in range(layers)],
+    }
+
+
+def dense_like(width, layers, hidden, vocab=32768):
+    """The dense decoder of the same width and depth whose feed-forward is as wide as a token's experts together."""
+    return dict(LLAMA3_8B, dim=width, n_layers=layers, n_heads=width // 128, n_kv_heads=8, head_dim=128, vocab_size=vocab,
+                hidden_dim=hidden, max_seq_len=131072)
+
+
+# sizes of the comparison: name -> (Lapevik arguments, feed-forward width of the dense decoder beside it)
+LAPEVIK_SIZES = {
+    "w2048": (dict(width=2048, layers=8, heads=16, kv_rank=192, q_rank=768, ssm_heads=64, state=128, groups=8, ff=1024, experts=16, top=4), 4096),
+    "w4096": (dict(width=4096, layers=8, heads=32, kv_rank=192, q_rank=1536, ssm_heads=128, state=128, groups=8, ff=1536, experts=32, top=4), 6144),
+}
+
+
+def compare_lapevik(args, device):
+    """Prefill and decode of the Lapevik design at sizes like a real model's layers, beside the dense decoder of equal
+    width, depth and active feed-forward width: one JSON line."""
+    out = {"compare": "lapevik", "dtype": args.dtype, "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens, "sizes": {}}
+    names = [args.size] if args.size else list(LAPEVIK_SIZES)
+    for name in names:
+        sizes, hidden = LAPEVIK_SIZES[name]
+        row = {}
+        for label, config in (("lapevik", lapevik_config(**sizes)), ("llama3_dense", dense_like(sizes["width"], sizes["layers"], hidden))):
+            if args.only and label != args.only:
+                continue
+            bench = ShapeBench(f"{label} {name}", config, None, args.dtype, args.page, args.graphs, device)
+            seconds = bench.prefill_run(args.prefill_tokens)
+            flops = bench.prefill_flops(args.prefill_tokens)
+            row[label] = {
+                "prefill_tok_s": round(args.prefill_tokens / seconds, 1), "prefill_ms": round(seconds * 1e3, 2),
+                "prefill_frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4), "active_matrix_params": bench.matrix_params,
+                "weight_gb": round(bench.weight_bytes / 1e9, 3),
+            }
+            for batch in sorted({1, args.batch}):
+                tok_s, ms = bench.decode_run(batch, args.context, args.steps, args.warmup)
+                row[label][f"decode_b{batch}_tok_s"] = round(tok_s, 1)
+                row[label][f"decode_b{batch}_ms"] = round(ms, 3)
+                row[label][f"decode_b{batch}_frac_of_all_weights"] = round(bench.step_bytes(batch, args.context) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            bench.close()
+        out["sizes"][name] = row
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -309,6 +378,9 @@ def main() -> int:
         "through the engine's scheduler (continuous batching, temperature 0.7, top-p 0.95)",
     )
     ap.add_argument("--new", type=int, default=512, help="tokens generated per request with --serve")
+    ap.add_argument("--compare", default=None, choices=["lapevik"], help="instead of the step benchmark: prefill and decode of another design beside the dense decoder of equal size")
+    ap.add_argument("--size", default=None, choices=sorted(LAPEVIK_SIZES), help="with --compare: one size only")
+    ap.add_argument("--only", default=None, choices=["lapevik", "llama3_dense"], help="with --compare: one of the two models only")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -317,6 +389,9 @@ def main() -> int:
     import torch
 
     device = torch.device("cuda:0")
+    if args.compare:
+        print(json.dumps(compare_lapevik(args, device)), flush=True)
+        return 0
     shape_name, shape = SHAPES[args.shape]
     if args.config:
         with open(args.config) as f:
