@@ -177,81 +177,96 @@ template <> struct Frag<float> {
   }
 };
 
-// A block of four wavefronts takes RT row tiles of one expert (they follow one another in the list) and 64 columns;
-// wavefront w the columns 16 w .. 16 w + 15 for all of the block's rows, so a weight tile is loaded once for RT
-// tiles of rows.  VEC: rows of a and W start at multiples of 16 bytes and K is a multiple of a lane's piece.
-template <typename T, int RT, bool GATED, bool VEC>
+// A block of four wavefronts, WR of them down the rows and 4 / WR along the columns, takes WR * RT row tiles of one
+// expert (they follow one another in the list, and an expert's tiles start at a multiple of that many) and
+// (4 / WR) * CT * 16 columns; a wavefront multiplies RT row tiles by CT column tiles, so each piece of a weight tile
+// it loads serves RT tiles of rows and each piece of rows CT tiles of columns.  Shapes in use: 1 x 1 tiles a
+// wavefront, four wavefronts along the columns (few rows an expert: many blocks stream the weights); 4 x 1 likewise;
+// 4 x 4 (4 x 2 with two weights) with the wavefronts 2 x 2 (many rows an expert).
+// VEC: rows of a and W start at multiples of 16 bytes and K is a multiple of a lane's piece.
+template <typename T, int RT, int CT, int WR, bool GATED, bool VEC>
 __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
                                                               const T* __restrict__ w0, const T* __restrict__ w1, long w_stride,
                                                               const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
                                                               int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+  constexpr int WC = 4 / WR;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
+  const int wave_r = wave / WC, wave_c = wave % WC;
   const int r = lane & 15, j = lane >> 4;
-  const int tile0 = blockIdx.x * RT;
+  const int block_tile0 = blockIdx.x * (WR * RT);
+  const int tile0 = block_tile0 + wave_r * RT;
   int expert;
   if (tile_expert) {
-    expert = tile0 < n_tiles ? tile_expert[tile0] : -1;
+    expert = block_tile0 < n_tiles ? tile_expert[block_tile0] : -1;
     if (expert < 0) return;
   } else {
     expert = blockIdx.z;
   }
-  const int n0 = blockIdx.y * 64 + wave * 16;
+  const int n0 = (blockIdx.y * WC + wave_c) * CT * 16;
   if (n0 >= N) return;
-  const int col = n0 + r;
-  const T* wrow0 = w0 + (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K;
-  const T* wrow1 = GATED ? w1 + (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K : nullptr;
+  const T* wrow0[CT];
+  const T* wrow1[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = n0 + ct * 16 + r;
+    const size_t at = (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K;
+    wrow0[ct] = w0 + at;
+    wrow1[ct] = GATED ? w1 + at : nullptr;
+  }
   const T* arow[RT];
   bool tile_live[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int tile = tile0 + rt;
-    // a tile of another expert, or beyond the rows, is left out (its rows belong to another block)
+    // a tile of another expert, or beyond the rows, is left out
     tile_live[rt] = tile_expert ? (tile < n_tiles && tile_expert[tile] == expert) : tile * TILE_ROWS < n_rows;
     const int row = tile * TILE_ROWS + r;
     long src = -1;
     if (tile_live[rt]) src = row_token ? row_token[row] : (row < n_rows ? row : -1);
     arow[rt] = src >= 0 ? a + (size_t)blockIdx.z * a_batch + (size_t)src * a_ld : nullptr;
   }
-  float4v acc0[RT], acc1[RT];
+  float4v acc0[RT][CT], acc1[RT][CT];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) acc0[rt] = acc1[rt] = (float4v){0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc0[rt][ct] = acc1[rt][ct] = (float4v){0.f, 0.f, 0.f, 0.f};
   constexpr int STEP = Frag<T>::K_STEP, PIECE = Frag<T>::PER_LANE;
   for (int k0 = 0; k0 < K; k0 += STEP) {
     const int k = k0 + j * PIECE;
     const int left = K - k;  // values of this lane's piece inside K
-    Frag<T> fw0, fw1, fa[RT];
-    if (VEC) {
-      if (left > 0) {
-        fw0.load16(wrow0 + k);
-        if (GATED) fw1.load16(wrow1 + k);
+    Frag<T> fw0[CT], fw1[CT], fa[RT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      if (VEC) {
+        if (left > 0) {
+          fw0[ct].load16(wrow0[ct] + k);
+          if (GATED) fw1[ct].load16(wrow1[ct] + k);
+        } else {
+          fw0[ct].zero();
+          if (GATED) fw1[ct].zero();
+        }
       } else {
-        fw0.zero();
-        if (GATED) fw1.zero();
-      }
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if (arow[rt] && left > 0)
-          fa[rt].load16(arow[rt] + k);
-        else
-          fa[rt].zero();
-      }
-    } else {
-      fw0.load_some(wrow0 + k, left);
-      if (GATED) fw1.load_some(wrow1 + k, left);
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if (arow[rt])
-          fa[rt].load_some(arow[rt] + k, left);
-        else
-          fa[rt].zero();
+        fw0[ct].load_some(wrow0[ct] + k, left);
+        if (GATED) fw1[ct].load_some(wrow1[ct] + k, left);
       }
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      acc0[rt] = Frag<T>::mma(fw0, fa[rt], acc0[rt]);
-      if (GATED) acc1[rt] = Frag<T>::mma(fw1, fa[rt], acc1[rt]);
+      if (!arow[rt] || left <= 0)
+        fa[rt].zero();
+      else if (VEC)
+        fa[rt].load16(arow[rt] + k);
+      else
+        fa[rt].load_some(arow[rt] + k, left);
     }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        acc0[rt][ct] = Frag<T>::mma(fw0[ct], fa[rt], acc0[rt][ct]);
+        if (GATED) acc1[rt][ct] = Frag<T>::mma(fw1[ct], fa[rt], acc1[rt][ct]);
+      }
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -260,35 +275,40 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
     if (!tile_expert && row >= n_rows) continue;
     const size_t base = (size_t)blockIdx.z * out_batch + (size_t)row * out_ld;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = n0 + 4 * j + i;
-      if (c >= N) continue;
-      float v = acc0[rt][i];
-      if (GATED) v = v / (1.f + expf(-v)) * acc1[rt][i];
-      if (out_dtype == CWM_F32)
-        ((float*)out)[base + c] = v;
-      else
-        ((bf16_t*)out)[base + c] = f32_to_bf16(v);
-    }
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = n0 + ct * 16 + 4 * j + i;
+        if (c >= N) continue;
+        float v = acc0[rt][ct][i];
+        if (GATED) v = v / (1.f + expf(-v)) * acc1[rt][ct][i];
+        if (out_dtype == CWM_F32)
+          ((float*)out)[base + c] = v;
+        else
+          ((bf16_t*)out)[base + c] = f32_to_bf16(v);
+      }
   }
 }
 
-template <typename T, int RT, bool GATED>
-static void launch_grouped(bool vec, dim3 grid, hipStream_t stream, const T* a, long a_ld, long a_batch, const int* row_token, const T* w0,
-                           const T* w1, long w_stride, const int* tile_expert, int n_tiles, void* out, int out_dtype, long out_ld,
-                           long out_batch, int n_rows, int N, int K) {
+template <typename T, int RT, int CT, int WR, bool GATED>
+static void launch_grouped(bool vec, int tiles, int n_batch, hipStream_t stream, const T* a, long a_ld, long a_batch, const int* row_token,
+                           const T* w0, const T* w1, long w_stride, const int* tile_expert, int n_tiles, void* out, int out_dtype,
+                           long out_ld, long out_batch, int n_rows, int N, int K) {
+  constexpr int block_tiles = WR * RT, block_cols = (4 / WR) * CT * 16;
+  dim3 grid((tiles + block_tiles - 1) / block_tiles, (N + block_cols - 1) / block_cols, n_batch);
   if (vec)
-    hipLaunchKernelGGL((grouped_product_kernel<T, RT, GATED, true>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1, w_stride,
-                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+    hipLaunchKernelGGL((grouped_product_kernel<T, RT, CT, WR, GATED, true>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1,
+                       w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
   else
-    hipLaunchKernelGGL((grouped_product_kernel<T, RT, GATED, false>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1, w_stride,
-                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+    hipLaunchKernelGGL((grouped_product_kernel<T, RT, CT, WR, GATED, false>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1,
+                       w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
 }
 
 // a: rows of K values, `a_ld` apart (row `row_token[row]` for list row `row` if a list is given; batch z starts
 // `a_batch` further).  w0 (and w1 for the gated form): [experts or batches][N][K], `w_stride` apart.  With
 // `tile_expert` the rows are the list's n_tiles * 16 and out is [rows][out_ld]; without, every batch z < n_batch
-// multiplies the same n_rows rows by its own weight into out + z * out_batch.
+// multiplies the same n_rows rows by its own weight into out + z * out_batch.  tiles_a_block: 1, 4 or 8 row tiles
+// a block (with a list, an expert's tiles start at a multiple of it).
 extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int dtype, const int* row_token, const void* w0, const void* w1,
                                    long w_stride, const int* tile_expert, int n_tiles, int n_batch, void* out, int out_dtype, long out_ld,
                                    long out_batch, int n_rows, int N, int K, int tiles_a_block, hipStream_t stream) {
@@ -301,24 +321,31 @@ extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int d
   const int piece = dtype == CWM_BF16 ? 8 : 4;
   const bool vec = K % piece == 0 && (a_ld * esize) % 16 == 0 && (a_batch * esize) % 16 == 0 && (w_stride * esize) % 16 == 0 &&
                    ((uintptr_t)a % 16) == 0 && ((uintptr_t)w0 % 16) == 0 && (!w1 || ((uintptr_t)w1 % 16) == 0);
-  // many rows an expert: four row tiles share each weight tile; few: one, so that more blocks stream the weights
-  CWM_REQUIRE(tiles_a_block == 1 || tiles_a_block == 4, "grouped_product: a block takes 1 or 4 row tiles");
-  const bool wide = tiles_a_block == 4;
-  const int rt = tiles_a_block;
-  dim3 grid((tiles + rt - 1) / rt, (N + 63) / 64, tile_expert ? 1 : n_batch);
-  CWM_REQUIRE(grid.y <= 65535, "grouped_product: too many columns");
-#define CWM_GROUPED(T, RT, GATED)                                                                                                      \
-  launch_grouped<T, RT, GATED>(vec, grid, stream, (const T*)a, a_ld, a_batch, row_token, (const T*)w0, (const T*)w1, w_stride, tile_expert, \
-                               n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K)
-  if (dtype == CWM_BF16) {
-    if (w1) { if (wide) CWM_GROUPED(bf16_t, 4, true); else CWM_GROUPED(bf16_t, 1, true); }
-    else    { if (wide) CWM_GROUPED(bf16_t, 4, false); else CWM_GROUPED(bf16_t, 1, false); }
-  } else if (dtype == CWM_F32) {
-    if (w1) { if (wide) CWM_GROUPED(float, 4, true); else CWM_GROUPED(float, 1, true); }
-    else    { if (wide) CWM_GROUPED(float, 4, false); else CWM_GROUPED(float, 1, false); }
-  } else {
+  CWM_REQUIRE(tiles_a_block == 1 || tiles_a_block == 4 || tiles_a_block == 8, "grouped_product: a block takes 1, 4 or 8 row tiles");
+  CWM_REQUIRE((N + 15) / 16 <= 65535, "grouped_product: too many columns");
+  const int nb = tile_expert ? 1 : n_batch;
+#define CWM_GROUPED(T, RT, CT, WR, GATED)                                                                                                 \
+  launch_grouped<T, RT, CT, WR, GATED>(vec, tiles, nb, stream, (const T*)a, a_ld, a_batch, row_token, (const T*)w0, (const T*)w1, w_stride, \
+                                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K)
+#define CWM_GROUPED_SHAPES(T)                                                   \
+  do {                                                                          \
+    if (w1) {                                                                   \
+      if (tiles_a_block == 8) CWM_GROUPED(T, 4, 2, 2, true);                    \
+      else if (tiles_a_block == 4) CWM_GROUPED(T, 4, 1, 1, true);               \
+      else CWM_GROUPED(T, 1, 1, 1, true);                                       \
+    } else {                                                                    \
+      if (tiles_a_block == 8) CWM_GROUPED(T, 4, 4, 2, false);                   \
+      else if (tiles_a_block == 4) CWM_GROUPED(T, 4, 1, 1, false);              \
+      else CWM_GROUPED(T, 1, 1, 1, false);                                      \
+    }                                                                           \
+  } while (0)
+  if (dtype == CWM_BF16)
+    CWM_GROUPED_SHAPES(bf16_t);
+  else if (dtype == CWM_F32)
+    CWM_GROUPED_SHAPES(float);
+  else
     return cwm_fail("grouped_product: unknown dtype %d", dtype);
-  }
+#undef CWM_GROUPED_SHAPES
 #undef CWM_GROUPED
   return cwm_launch_status("grouped_product");
 }

@@ -105,10 +105,17 @@ extern "C" int cwm_conv_silu(const void* in, long in_ld, int dtype, const float*
   return cwm_launch_status("conv_silu");
 }
 
-// One block per (tile of P, head, sequence).  Thread (p, s) holds rows s, s + split, s + 2 split, ... of column p of
-// the head's state (split a power of two, the split lanes of one column adjacent in a wavefront), walks the
-// sequence's tokens of this step in order, and the split lanes add their parts of y_t[p] by shuffles in a fixed
-// order.  The state is read once before and written once after the walk.
+// One block per (tile of P, head, sequence).  Thread (p, s) holds 16 rows of column p of the head's state: with
+// `split` lanes a column (a power of two, adjacent in a wavefront), lane s has rows 4 (s + q split) + j, q, j < 4,
+// so that its B and C values are four 16-byte pieces of LDS.  The block walks the sequence's tokens of this step in
+// order, SCAN_TC at a time: while it computes on one chunk from LDS (B, C and the tile's x as float32, the step
+// sizes and decays computed once a token), the next chunk's values are already on their way into registers.  The
+// split lanes add their parts of y_t[p] by shuffles in a fixed order.  The state is read once before and written
+// once after the walk; what a token's result is made of, and in which order, does not depend on how the
+// sequence is cut into steps.
+#define SCAN_TC 16  // tokens of a chunk
+#define SCAN_PF 36  // most values of a chunk that one thread fetches
+
 template <typename T>
 __global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt_raw,
                                                              long dt_ld, const float* __restrict__ dt_bias,
@@ -116,52 +123,118 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict
                                                              float* state, long state_ld, const int* __restrict__ slots,
                                                              const int* __restrict__ cu_q, float* __restrict__ y, int heads, int P,
                                                              int N, int groups, int split, int n_slots) {
+  extern __shared__ float lds[];
   const int h = blockIdx.y;
   const int b = blockIdx.z;
   const int cols = blockDim.x / split;
   const int s = threadIdx.x % split;
-  const int p = blockIdx.x * cols + threadIdx.x / split;
+  const int col = threadIdx.x / split;
+  const int p0 = blockIdx.x * cols;
+  const int p = p0 + col;
   const bool live = p < P;
-  const int pc = live ? p : P - 1;  // idle threads follow along (the shuffles need every lane) and store nothing
   const int g = h / (heads / groups);
   const int inner = heads * P;
+  const int NB = SCAN_ROWS * split;      // rows of B (and of C) in LDS, zeros from N on
+  const int row = 2 * NB + cols;         // a token's values in LDS: B, C, the tile's x
+  float* dtv = lds + SCAN_TC * row;      // the chunk's step sizes
+  float* av = dtv + SCAN_TC;             // and decays
   const int slot = slots[b];
   float* st = (slot >= 0 && slot < n_slots) ? state + (size_t)slot * state_ld + (size_t)h * N * P : nullptr;
   float S[SCAN_ROWS];
 #pragma unroll
   for (int i = 0; i < SCAN_ROWS; ++i) {
-    const int n = s + i * split;
-    S[i] = (st && n < N) ? st[(size_t)n * P + pc] : 0.f;
+    const int n = 4 * (s + (i >> 2) * split) + (i & 3);
+    S[i] = (st && live && n < N) ? st[(size_t)n * P + p] : 0.f;
   }
   const float bias = dt_bias[h];
   const float rate = -expf(a_log[h]);
   const float skip = d_skip[h];
   const int t0 = cu_q[b], t1 = cu_q[b + 1];
-  for (int t = t0; t < t1; ++t) {
-    const T* row = xbc + (size_t)t * xbc_ld;
-    const float z = Elem<T>::load(dt_raw + (size_t)t * dt_ld + h) + bias;
-    const float dt = z > 20.f ? z : log1pf(expf(z));
-    const float a = expf(rate * dt);
-    const float x = Elem<T>::load(row + (size_t)h * P + pc);
-    const float dx = dt * x;
-    const T* Bt = row + inner + (size_t)g * N;
-    const T* Ct = Bt + (size_t)groups * N;
-    float acc = 0.f;
+  const int total = SCAN_TC * row;
+
+  float pf[SCAN_PF];
+  float pf_dt = 0.f, pf_a = 0.f;
+  auto fetch = [&](int start) {  // the chunk that starts at token `start`, into registers
 #pragma unroll
-    for (int i = 0; i < SCAN_ROWS; ++i) {
-      const int n = s + i * split;
-      if (n < N) {
-        S[i] = a * S[i] + Elem<T>::load(Bt + n) * dx;
-        acc += S[i] * Elem<T>::load(Ct + n);
+    for (int k = 0; k < SCAN_PF; ++k) {
+      const int idx = threadIdx.x + k * 256;
+      float v = 0.f;
+      if (idx < total) {
+        const int tc = idx / row, e = idx - tc * row;
+        const int t = start + tc;
+        if (t < t1) {
+          const T* src = xbc + (size_t)t * xbc_ld;
+          if (e < NB) {
+            if (e < N) v = Elem<T>::load(src + inner + (size_t)g * N + e);
+          } else if (e < 2 * NB) {
+            if (e - NB < N) v = Elem<T>::load(src + inner + (size_t)(groups + g) * N + (e - NB));
+          } else if (p0 + e - 2 * NB < P) {
+            v = Elem<T>::load(src + (size_t)h * P + p0 + (e - 2 * NB));
+          }
+        }
+      }
+      pf[k] = v;
+    }
+    if (threadIdx.x < SCAN_TC) {
+      const int t = start + threadIdx.x;
+      if (t < t1) {
+        const float z = Elem<T>::load(dt_raw + (size_t)t * dt_ld + h) + bias;
+        pf_dt = z > 20.f ? z : log1pf(expf(z));
+        pf_a = expf(rate * pf_dt);
       }
     }
-    for (int off = 1; off < split; off <<= 1) acc += __shfl_xor(acc, off, CWM_WAVE);
-    if (live && s == 0) y[(size_t)t * inner + (size_t)h * P + p] = acc + skip * x;
+  };
+  auto stage = [&]() {  // registers -> LDS
+#pragma unroll
+    for (int k = 0; k < SCAN_PF; ++k) {
+      const int idx = threadIdx.x + k * 256;
+      if (idx < total) lds[idx] = pf[k];
+    }
+    if (threadIdx.x < SCAN_TC) {
+      dtv[threadIdx.x] = pf_dt;
+      av[threadIdx.x] = pf_a;
+    }
+  };
+
+  fetch(t0);
+  stage();
+  __syncthreads();
+  for (int start = t0; start < t1; start += SCAN_TC) {
+    const bool more = start + SCAN_TC < t1;
+    if (more) fetch(start + SCAN_TC);
+    const int n_here = min(SCAN_TC, t1 - start);
+    for (int tc = 0; tc < n_here; ++tc) {
+      const float* tok = lds + tc * row;
+      const float dt = dtv[tc], a = av[tc];
+      const float x = tok[2 * NB + col];
+      const float dx = dt * x;
+      float acc = 0.f;
+#pragma unroll
+      for (int q = 0; q < SCAN_ROWS / 4; ++q) {
+        const float4 Bq = *(const float4*)(tok + 4 * (s + q * split));
+        const float4 Cq = *(const float4*)(tok + NB + 4 * (s + q * split));
+        S[4 * q + 0] = a * S[4 * q + 0] + Bq.x * dx;
+        S[4 * q + 1] = a * S[4 * q + 1] + Bq.y * dx;
+        S[4 * q + 2] = a * S[4 * q + 2] + Bq.z * dx;
+        S[4 * q + 3] = a * S[4 * q + 3] + Bq.w * dx;
+        acc += S[4 * q + 0] * Cq.x;
+        acc += S[4 * q + 1] * Cq.y;
+        acc += S[4 * q + 2] * Cq.z;
+        acc += S[4 * q + 3] * Cq.w;
+      }
+      for (int off = 1; off < split; off <<= 1) acc += __shfl_xor(acc, off, CWM_WAVE);
+      if (live && s == 0) y[(size_t)(start + tc) * inner + (size_t)h * P + p] = acc + skip * x;
+    }
+    __syncthreads();
+    if (more) {
+      stage();
+      __syncthreads();
+    }
   }
   if (st && live) {
 #pragma unroll
     for (int i = 0; i < SCAN_ROWS; ++i) {
-      const int n = s + i * split;
+      const int n = 4 * (s + (i >> 2) * split) + (i & 3);
       if (n < N) st[(size_t)n * P + p] = S[i];
     }
   }
@@ -182,11 +255,14 @@ extern "C" int cwm_selective_scan(const void* xbc, long xbc_ld, const void* dt_r
   while (split * SCAN_ROWS < N) split <<= 1;  // 1, 2, 4, 8 or 16 lanes a column
   const int cols = 256 / split;
   dim3 grid((P + cols - 1) / cols, heads, n_seqs);
+  const int row = 2 * SCAN_ROWS * split + cols;
+  const size_t lds_bytes = (size_t)(SCAN_TC * row + 2 * SCAN_TC) * sizeof(float);
+  CWM_REQUIRE(SCAN_TC * row <= SCAN_PF * 256, "selective_scan: a chunk of %d values is more than the threads fetch", SCAN_TC * row);
   if (dtype == CWM_BF16)
-    hipLaunchKernelGGL(selective_scan_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)xbc, xbc_ld, (const bf16_t*)dt_raw, dt_ld,
+    hipLaunchKernelGGL(selective_scan_kernel<bf16_t>, grid, dim3(256), lds_bytes, stream, (const bf16_t*)xbc, xbc_ld, (const bf16_t*)dt_raw, dt_ld,
                        dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots);
   else if (dtype == CWM_F32)
-    hipLaunchKernelGGL(selective_scan_kernel<float>, grid, dim3(256), 0, stream, (const float*)xbc, xbc_ld, (const float*)dt_raw, dt_ld,
+    hipLaunchKernelGGL(selective_scan_kernel<float>, grid, dim3(256), lds_bytes, stream, (const float*)xbc, xbc_ld, (const float*)dt_raw, dt_ld,
                        dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots);
   else
     return cwm_fail("selective_scan: unknown dtype %d", dtype);

@@ -14,7 +14,8 @@ from . import build as _build
 MAX_ROUTE_TOP = 16  # csrc/routed.hip: ROUTE_MAX_TOP
 MAX_EXPERTS = 256  # csrc/routed.hip: ROUTE_MAX_EXPERTS
 TILE_ROWS = 16  # rows of a tile of the grouped product
-WIDE_ROWS_AN_EXPERT = 64  # from so many rows an expert (on average) a block takes four row tiles
+MEDIUM_ROWS = 64  # from so many rows an expert (on average) a block of the grouped product takes 4 row tiles,
+WIDE_ROWS = 256  # and from so many, 8
 
 
 def _base():
@@ -52,6 +53,10 @@ class ExpertGroups:
     top: int
 
 
+def _tiles_a_block(rows: float) -> int:
+    return 8 if rows >= WIDE_ROWS else 4 if rows >= MEDIUM_ROWS else 1
+
+
 def group_by_expert(chosen: torch.Tensor, n_experts: int) -> ExpertGroups:
     """Group the pairs of `chosen` (int32 [T, top]) by expert.  The lists have a size that depends on T, top and
     the number of experts alone, so no count has to come to the host."""
@@ -64,7 +69,7 @@ def group_by_expert(chosen: torch.Tensor, n_experts: int) -> ExpertGroups:
         raise KernelError(f"{n_experts} experts: the kernel takes up to {MAX_EXPERTS}")
     n, top = chosen.shape
     pairs = n * top
-    align = 4 if pairs >= WIDE_ROWS_AN_EXPERT * n_experts else 1
+    align = _tiles_a_block(pairs / n_experts)
     n_tiles = -(-pairs // TILE_ROWS) + n_experts * align
     lists = torch.empty(n_tiles * TILE_ROWS + pairs + n_tiles, dtype=torch.int32, device=chosen.device)
     a, b = n_tiles * TILE_ROWS, n_tiles * TILE_ROWS + pairs
@@ -169,7 +174,7 @@ def absorb_queries(q: torch.Tensor, lead: int, weight: torch.Tensor) -> torch.Te
     if lead:
         out[:, :, :lead].copy_(q[:, :, :lead])
     if n_tokens:
-        tiles = 4 if n_tokens >= WIDE_ROWS_AN_EXPERT else 1
+        tiles = _tiles_a_block(n_tokens)
         _grouped(q.view(-1)[lead:], heads * width, width, None, weight, None, out.view(-1)[lead:], heads * (lead + n), lead + n, n_tokens, heads, tiles)
     return out
 
@@ -184,6 +189,6 @@ def expand_values(mixed: torch.Tensor, lead: int, weight: torch.Tensor) -> torch
     v = weight.shape[1]
     out = torch.empty((n_tokens, heads * v), dtype=mixed.dtype, device=mixed.device)
     if n_tokens:
-        tiles = 4 if n_tokens >= WIDE_ROWS_AN_EXPERT else 1
+        tiles = _tiles_a_block(n_tokens)
         _grouped(mixed.view(-1)[lead:], heads * width, width, None, weight, None, out, heads * v, v, n_tokens, heads, tiles)
     return out

@@ -172,7 +172,7 @@ def test_route_top(n_experts, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n_tokens,dim,hidden,n_experts,top", [(1, 64, 32, 8, 4), (9, 192, 96, 8, 4), (200, 72, 40, 3, 2), (300, 64, 50, 4, 1), (33, 100, 36, 16, 3)])
+@pytest.mark.parametrize("n_tokens,dim,hidden,n_experts,top", [(1, 64, 32, 8, 4), (9, 192, 96, 8, 4), (200, 72, 40, 3, 2), (300, 64, 50, 4, 1), (33, 100, 36, 16, 3), (1200, 64, 48, 2, 1), (700, 40, 72, 3, 2)])
 def test_routed_experts_pipeline(dtype, n_tokens, dim, hidden, n_experts, top):
     """Grouping, both grouped products and the weighted sum, against one product per pair; sizes that are no
     multiple of a lane's piece take the kernels' element-wise loads."""
@@ -203,7 +203,7 @@ def test_routed_experts_pipeline(dtype, n_tokens, dim, hidden, n_experts, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n_tokens,heads,lead,d,n", [(1, 6, 16, 64, 64), (70, 3, 8, 24, 40), (5, 2, 6, 10, 30), (130, 4, 0, 32, 16)])
+@pytest.mark.parametrize("n_tokens,heads,lead,d,n", [(1, 6, 16, 64, 64), (70, 3, 8, 24, 40), (5, 2, 6, 10, 30), (130, 4, 0, 32, 16), (300, 2, 16, 64, 80)])
 def test_products_per_head(dtype, n_tokens, heads, lead, d, n):
     from cwm_amd import ops
 
