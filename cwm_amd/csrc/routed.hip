@@ -232,10 +232,10 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) acc0[rt][ct] = acc1[rt][ct] = (float4v){0.f, 0.f, 0.f, 0.f};
   constexpr int STEP = Frag<T>::K_STEP, PIECE = Frag<T>::PER_LANE;
-  for (int k0 = 0; k0 < K; k0 += STEP) {
+  // two sets of operands: while one is multiplied, the loads of the next step are in flight
+  auto load_set = [&](Frag<T> (&fw0)[CT], Frag<T> (&fw1)[CT], Frag<T> (&fa)[RT], int k0) {
     const int k = k0 + j * PIECE;
     const int left = K - k;  // values of this lane's piece inside K
-    Frag<T> fw0[CT], fw1[CT], fa[RT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       if (VEC) {
@@ -260,6 +260,8 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
       else
         fa[rt].load_some(arow[rt] + k, left);
     }
+  };
+  auto multiply = [&](const Frag<T> (&fw0)[CT], const Frag<T> (&fw1)[CT], const Frag<T> (&fa)[RT]) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -267,6 +269,14 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
         acc0[rt][ct] = Frag<T>::mma(fw0[ct], fa[rt], acc0[rt][ct]);
         if (GATED) acc1[rt][ct] = Frag<T>::mma(fw1[ct], fa[rt], acc1[rt][ct]);
       }
+  };
+  Frag<T> w0a[CT], w1a[CT], ra[RT], w0b[CT], w1b[CT], rb[RT];
+  load_set(w0a, w1a, ra, 0);
+  for (int k0 = 0; k0 < K; k0 += 2 * STEP) {
+    load_set(w0b, w1b, rb, k0 + STEP);  // beyond K: zeros
+    multiply(w0a, w1a, ra);
+    load_set(w0a, w1a, ra, k0 + 2 * STEP);
+    multiply(w0b, w1b, rb);
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {

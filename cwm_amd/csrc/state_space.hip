@@ -8,10 +8,12 @@
 //       dt = softplus(dt_raw + dt_bias[h]);  a = exp(-exp(A_log[h]) * dt)
 //       S <- a S + dt B_t x_t^T;   y_t = S^T C_t + D[h] x_t
 //     with x_t [P], B_t and C_t [N] from the convolution's output row [x: heads * P | B: groups * N | C: groups * N].
+//     A head's state lies in memory in the order its threads hold it (see the kernel), padded to 16 * split rows.
 //
 // Both are exact under any cut of a sequence into portions: a portion starts from the state as the previous one
 // left it and performs the same operations in the same order as the whole sequence would.
 #include "common.h"
+#include <type_traits>
 
 CWM_DEFINE_ERROR_API
 
@@ -20,6 +22,12 @@ CWM_DEFINE_ERROR_API
 
 extern "C" int cwm_conv_max_taps() { return CONV_MAX_TAPS; }
 extern "C" int cwm_scan_max_state() { return SCAN_ROWS * 16; }
+// lanes that share a column of a head's state of N rows: 1, 2, 4, 8 or 16; the head's state takes SCAN_ROWS * split * P floats
+extern "C" int cwm_scan_split(int N) {
+  int split = 1;
+  while (split * SCAN_ROWS < N) split <<= 1;
+  return split;
+}
 
 __device__ __forceinline__ float silu_f32(float z) { return z / (1.f + expf(-z)); }
 
@@ -108,25 +116,28 @@ extern "C" int cwm_conv_silu(const void* in, long in_ld, int dtype, const float*
 // One block per (tile of P, head, sequence).  Thread (p, s) holds 16 rows of column p of the head's state: with
 // `split` lanes a column (a power of two, adjacent in a wavefront), lane s has rows 4 (s + q split) + j, q, j < 4,
 // so that its B and C values are four 16-byte pieces of LDS.  The block walks the sequence's tokens of this step in
-// order, SCAN_TC at a time: while it computes on one chunk from LDS (B, C and the tile's x as float32, the step
+// order, a chunk of up to 16 at a time: while it computes on one chunk from LDS (B, C and the tile's x as float32, the step
 // sizes and decays computed once a token), the next chunk's values are already on their way into registers.  The
 // split lanes add their parts of y_t[p] by shuffles in a fixed order.  The state is read once before and written
 // once after the walk; what a token's result is made of, and in which order, does not depend on how the
 // sequence is cut into steps.
-#define SCAN_TC 16  // tokens of a chunk
 #define SCAN_PF 36  // most values of a chunk that one thread fetches
 
-template <typename T>
-__global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt_raw,
-                                                             long dt_ld, const float* __restrict__ dt_bias,
-                                                             const float* __restrict__ a_log, const float* __restrict__ d_skip,
-                                                             float* state, long state_ld, const int* __restrict__ slots,
-                                                             const int* __restrict__ cu_q, float* __restrict__ y, int heads, int P,
-                                                             int N, int groups, int split, int n_slots) {
+// THREADS a block, TC tokens a chunk.  VEC: the rows of xbc start at multiples of 16 bytes and N and P are multiples
+// of the values in 16 bytes, so a chunk is fetched in pieces of 16 bytes; otherwise value by value.
+#define SCAN_PFV 6  // most 16-byte pieces of a chunk that one thread fetches
+
+template <typename T, int THREADS, int TC, bool VEC>
+__global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt_raw,
+                                                                 long dt_ld, const float* __restrict__ dt_bias,
+                                                                 const float* __restrict__ a_log, const float* __restrict__ d_skip,
+                                                                 float* state, long state_ld, const int* __restrict__ slots,
+                                                                 const int* __restrict__ cu_q, float* __restrict__ y, int heads, int P,
+                                                                 int N, int groups, int split, int n_slots) {
   extern __shared__ float lds[];
   const int h = blockIdx.y;
   const int b = blockIdx.z;
-  const int cols = blockDim.x / split;
+  const int cols = THREADS / split;
   const int s = threadIdx.x % split;
   const int col = threadIdx.x / split;
   const int p0 = blockIdx.x * cols;
@@ -134,36 +145,66 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict
   const bool live = p < P;
   const int g = h / (heads / groups);
   const int inner = heads * P;
-  const int NB = SCAN_ROWS * split;      // rows of B (and of C) in LDS, zeros from N on
-  const int row = 2 * NB + cols;         // a token's values in LDS: B, C, the tile's x
-  float* dtv = lds + SCAN_TC * row;      // the chunk's step sizes
-  float* av = dtv + SCAN_TC;             // and decays
+  const int NB = SCAN_ROWS * split;  // rows of B (and of C) in LDS, zeros from N on
+  const int row = 2 * NB + cols;     // a token's values in LDS: B, C, the tile's x
+  float* dtv = lds + TC * row;       // the chunk's step sizes
+  float* av = dtv + TC;              // and decays
   const int slot = slots[b];
-  float* st = (slot >= 0 && slot < n_slots) ? state + (size_t)slot * state_ld + (size_t)h * N * P : nullptr;
+  // A head's state in memory, as its threads hold it: [q][p][s][j] for row 4 (s + q split) + j of column p, so that a
+  // thread's four rows are 16 bytes and the split lanes of a column lie side by side (rows from N on stay zero).
+  float* st = (slot >= 0 && slot < n_slots) ? state + (size_t)slot * state_ld + (size_t)h * SCAN_ROWS * split * P : nullptr;
   float S[SCAN_ROWS];
 #pragma unroll
-  for (int i = 0; i < SCAN_ROWS; ++i) {
-    const int n = 4 * (s + (i >> 2) * split) + (i & 3);
-    S[i] = (st && live && n < N) ? st[(size_t)n * P + p] : 0.f;
+  for (int q = 0; q < SCAN_ROWS / 4; ++q) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (st && live) v = *(const float4*)(st + (((size_t)q * P + p) * split + s) * 4);
+    S[4 * q + 0] = v.x, S[4 * q + 1] = v.y, S[4 * q + 2] = v.z, S[4 * q + 3] = v.w;
   }
   const float bias = dt_bias[h];
   const float rate = -expf(a_log[h]);
   const float skip = d_skip[h];
   const int t0 = cu_q[b], t1 = cu_q[b + 1];
-  const int total = SCAN_TC * row;
 
-  float pf[SCAN_PF];
+  constexpr int U = 16 / sizeof(T);  // values in 16 bytes
+  float pf[VEC ? 1 : SCAN_PF];
+  uint4 pfv[VEC ? SCAN_PFV : 1];
+  int pfv_at[VEC ? SCAN_PFV : 1];  // where in LDS each piece goes (-1: nowhere)
   float pf_dt = 0.f, pf_a = 0.f;
   auto fetch = [&](int start) {  // the chunk that starts at token `start`, into registers
+    const int n_tok = min(TC, t1 - start);  // what lies behind the sequence's end is not read (nor used)
+    if constexpr (VEC) {
+      const int pieces = row / U;  // of one token
+      int tc = threadIdx.x / pieces, e = threadIdx.x - tc * pieces;
+      const int step_tc = THREADS / pieces, step_e = THREADS - step_tc * pieces;
 #pragma unroll
-    for (int k = 0; k < SCAN_PF; ++k) {
-      const int idx = threadIdx.x + k * 256;
-      float v = 0.f;
-      if (idx < total) {
-        const int tc = idx / row, e = idx - tc * row;
-        const int t = start + tc;
-        if (t < t1) {
-          const T* src = xbc + (size_t)t * xbc_ld;
+      for (int k = 0; k < SCAN_PFV; ++k) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        pfv_at[k] = tc < TC ? tc * row + e * U : -1;
+        if (tc < n_tok) {
+          const T* src = xbc + (size_t)(start + tc) * xbc_ld;
+          const int at = e * U;
+          if (at < NB) {
+            if (at < N) v = *(const uint4*)(src + inner + (size_t)g * N + at);
+          } else if (at < 2 * NB) {
+            if (at - NB < N) v = *(const uint4*)(src + inner + (size_t)(groups + g) * N + (at - NB));
+          } else if (p0 + at - 2 * NB < P) {
+            v = *(const uint4*)(src + (size_t)h * P + p0 + (at - 2 * NB));
+          }
+        }
+        pfv[k] = v;
+        tc += step_tc;
+        e += step_e;
+        if (e >= pieces) e -= pieces, ++tc;
+      }
+    } else {
+      const int total = n_tok * row;
+      int tc = 0, e = threadIdx.x;  // this thread's k-th value, number threadIdx.x + k * THREADS of the chunk, is value e of token tc
+      while (e >= row) e -= row, ++tc;
+#pragma unroll
+      for (int k = 0; k < SCAN_PF; ++k) {
+        float v = 0.f;
+        if (tc * row + e < total) {
+          const T* src = xbc + (size_t)(start + tc) * xbc_ld;
           if (e < NB) {
             if (e < N) v = Elem<T>::load(src + inner + (size_t)g * N + e);
           } else if (e < 2 * NB) {
@@ -172,10 +213,12 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict
             v = Elem<T>::load(src + (size_t)h * P + p0 + (e - 2 * NB));
           }
         }
+        pf[k] = v;
+        e += THREADS;
+        while (e >= row) e -= row, ++tc;
       }
-      pf[k] = v;
     }
-    if (threadIdx.x < SCAN_TC) {
+    if (threadIdx.x < TC) {
       const int t = start + threadIdx.x;
       if (t < t1) {
         const float z = Elem<T>::load(dt_raw + (size_t)t * dt_ld + h) + bias;
@@ -185,46 +228,89 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict
     }
   };
   auto stage = [&]() {  // registers -> LDS
+    if constexpr (VEC) {
 #pragma unroll
-    for (int k = 0; k < SCAN_PF; ++k) {
-      const int idx = threadIdx.x + k * 256;
-      if (idx < total) lds[idx] = pf[k];
+      for (int k = 0; k < SCAN_PFV; ++k) {
+        if (pfv_at[k] < 0) continue;
+        float* dst = lds + pfv_at[k];
+        if constexpr (sizeof(T) == 4) {
+          *(uint4*)dst = pfv[k];
+        } else {
+          const uint32_t w[4] = {pfv[k].x, pfv[k].y, pfv[k].z, pfv[k].w};
+          *(float4*)dst = make_float4(__uint_as_float(w[0] << 16), __uint_as_float(w[0] & 0xffff0000u), __uint_as_float(w[1] << 16),
+                                      __uint_as_float(w[1] & 0xffff0000u));
+          *(float4*)(dst + 4) = make_float4(__uint_as_float(w[2] << 16), __uint_as_float(w[2] & 0xffff0000u), __uint_as_float(w[3] << 16),
+                                            __uint_as_float(w[3] & 0xffff0000u));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < SCAN_PF; ++k) {
+        const int idx = threadIdx.x + k * THREADS;
+        if (idx < TC * row) lds[idx] = pf[k];
+      }
     }
-    if (threadIdx.x < SCAN_TC) {
+    if (threadIdx.x < TC) {
       dtv[threadIdx.x] = pf_dt;
       av[threadIdx.x] = pf_a;
+    }
+  };
+  // One chunk from LDS.  The walk itself holds no wait on another lane: every token leaves its lane's part of y in
+  // a register, and the parts of the whole chunk are added across the split lanes afterwards, side by side.  A full
+  // chunk runs without a condition in it, so that a token's reads from LDS can start while the one before computes.
+  auto walk = [&](auto full_tag, int start, int n_here) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    float part[TC], xs[TC];
+#pragma unroll
+    for (int tc = 0; tc < TC; ++tc) {
+      part[tc] = 0.f;
+      xs[tc] = 0.f;
+      if (FULL || tc < n_here) {
+        const float* tok = lds + tc * row;
+        const float a = av[tc];
+        const float x = tok[2 * NB + col];
+        const float dx = dtv[tc] * x;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < SCAN_ROWS / 4; ++q) {
+          const float4 Bq = *(const float4*)(tok + 4 * (s + q * split));
+          const float4 Cq = *(const float4*)(tok + NB + 4 * (s + q * split));
+          S[4 * q + 0] = a * S[4 * q + 0] + Bq.x * dx;
+          S[4 * q + 1] = a * S[4 * q + 1] + Bq.y * dx;
+          S[4 * q + 2] = a * S[4 * q + 2] + Bq.z * dx;
+          S[4 * q + 3] = a * S[4 * q + 3] + Bq.w * dx;
+          acc[0] += S[4 * q + 0] * Cq.x;
+          acc[1] += S[4 * q + 1] * Cq.y;
+          acc[2] += S[4 * q + 2] * Cq.z;
+          acc[3] += S[4 * q + 3] * Cq.w;
+        }
+        part[tc] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        xs[tc] = x;
+      }
+    }
+    for (int off = 1; off < split; off <<= 1) {
+#pragma unroll
+      for (int tc = 0; tc < TC; ++tc)
+        if (FULL || tc < n_here) part[tc] += __shfl_xor(part[tc], off, CWM_WAVE);
+    }
+    if (live && s == 0) {
+#pragma unroll
+      for (int tc = 0; tc < TC; ++tc)
+        if (FULL || tc < n_here) y[(size_t)(start + tc) * inner + (size_t)h * P + p] = part[tc] + skip * xs[tc];
     }
   };
 
   fetch(t0);
   stage();
   __syncthreads();
-  for (int start = t0; start < t1; start += SCAN_TC) {
-    const bool more = start + SCAN_TC < t1;
-    if (more) fetch(start + SCAN_TC);
-    const int n_here = min(SCAN_TC, t1 - start);
-    for (int tc = 0; tc < n_here; ++tc) {
-      const float* tok = lds + tc * row;
-      const float dt = dtv[tc], a = av[tc];
-      const float x = tok[2 * NB + col];
-      const float dx = dt * x;
-      float acc = 0.f;
-#pragma unroll
-      for (int q = 0; q < SCAN_ROWS / 4; ++q) {
-        const float4 Bq = *(const float4*)(tok + 4 * (s + q * split));
-        const float4 Cq = *(const float4*)(tok + NB + 4 * (s + q * split));
-        S[4 * q + 0] = a * S[4 * q + 0] + Bq.x * dx;
-        S[4 * q + 1] = a * S[4 * q + 1] + Bq.y * dx;
-        S[4 * q + 2] = a * S[4 * q + 2] + Bq.z * dx;
-        S[4 * q + 3] = a * S[4 * q + 3] + Bq.w * dx;
-        acc += S[4 * q + 0] * Cq.x;
-        acc += S[4 * q + 1] * Cq.y;
-        acc += S[4 * q + 2] * Cq.z;
-        acc += S[4 * q + 3] * Cq.w;
-      }
-      for (int off = 1; off < split; off <<= 1) acc += __shfl_xor(acc, off, CWM_WAVE);
-      if (live && s == 0) y[(size_t)(start + tc) * inner + (size_t)h * P + p] = acc + skip * x;
-    }
+  for (int start = t0; start < t1; start += TC) {
+    const bool more = start + TC < t1;
+    if (more) fetch(start + TC);
+    const int n_here = min(TC, t1 - start);
+    if (n_here == TC)
+      walk(std::true_type{}, start, TC);
+    else
+      walk(std::false_type{}, start, n_here);
     __syncthreads();
     if (more) {
       stage();
@@ -233,11 +319,20 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(const T* __restrict
   }
   if (st && live) {
 #pragma unroll
-    for (int i = 0; i < SCAN_ROWS; ++i) {
-      const int n = 4 * (s + (i >> 2) * split) + (i & 3);
-      if (n < N) st[(size_t)n * P + p] = S[i];
-    }
+    for (int q = 0; q < SCAN_ROWS / 4; ++q)
+      *(float4*)(st + (((size_t)q * P + p) * split + s) * 4) = make_float4(S[4 * q + 0], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
   }
+}
+
+template <typename T, bool VEC>
+static void launch_scan(dim3 grid, int split, hipStream_t stream, const void* xbc, long xbc_ld, const void* dt_raw, long dt_ld,
+                        const float* dt_bias, const float* a_log, const float* d_skip, float* state, long state_ld, const int* slots,
+                        const int* cu_q, float* y, int heads, int P, int N, int groups, int n_slots) {
+  constexpr int THREADS = 256, TC = 16;
+  const int row = 2 * SCAN_ROWS * split + THREADS / split;
+  const size_t lds_bytes = (size_t)(TC * row + 2 * TC) * sizeof(float);
+  hipLaunchKernelGGL((selective_scan_kernel<T, THREADS, TC, VEC>), grid, dim3(THREADS), lds_bytes, stream, (const T*)xbc, xbc_ld,
+                     (const T*)dt_raw, dt_ld, dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots);
 }
 
 extern "C" int cwm_selective_scan(const void* xbc, long xbc_ld, const void* dt_raw, long dt_ld, int dtype, const float* dt_bias,
@@ -248,23 +343,26 @@ extern "C" int cwm_selective_scan(const void* xbc, long xbc_ld, const void* dt_r
   CWM_REQUIRE(heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0, "selective_scan: bad sizes");
   CWM_REQUIRE(N <= SCAN_ROWS * 16, "selective_scan: a state of %d rows, the kernel takes up to %d", N, SCAN_ROWS * 16);
   CWM_REQUIRE(xbc_ld >= (long)heads * P + 2L * groups * N && dt_ld >= heads, "selective_scan: rows too short");
-  CWM_REQUIRE((long)heads * N * P <= state_ld, "selective_scan: the state row is too short");
   CWM_REQUIRE(heads <= 65535 && n_seqs <= 65535, "selective_scan: too many heads or sequences for one launch");
+  const int split = cwm_scan_split(N);
+  CWM_REQUIRE((long)heads * SCAN_ROWS * split * P <= state_ld && state_ld % 4 == 0 && ((uintptr_t)state % 16) == 0,
+              "selective_scan: the state row is too short or not a multiple of 16 bytes");
   if (n_tokens == 0 || n_seqs == 0) return 0;
-  int split = 1;
-  while (split * SCAN_ROWS < N) split <<= 1;  // 1, 2, 4, 8 or 16 lanes a column
   const int cols = 256 / split;
-  dim3 grid((P + cols - 1) / cols, heads, n_seqs);
   const int row = 2 * SCAN_ROWS * split + cols;
-  const size_t lds_bytes = (size_t)(SCAN_TC * row + 2 * SCAN_TC) * sizeof(float);
-  CWM_REQUIRE(SCAN_TC * row <= SCAN_PF * 256, "selective_scan: a chunk of %d values is more than the threads fetch", SCAN_TC * row);
-  if (dtype == CWM_BF16)
-    hipLaunchKernelGGL(selective_scan_kernel<bf16_t>, grid, dim3(256), lds_bytes, stream, (const bf16_t*)xbc, xbc_ld, (const bf16_t*)dt_raw, dt_ld,
-                       dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots);
-  else if (dtype == CWM_F32)
-    hipLaunchKernelGGL(selective_scan_kernel<float>, grid, dim3(256), lds_bytes, stream, (const float*)xbc, xbc_ld, (const float*)dt_raw, dt_ld,
-                       dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots);
-  else
+  CWM_REQUIRE(16 * row <= SCAN_PF * 256, "selective_scan: a chunk of tokens does not fit the threads' registers");
+  dim3 grid((P + cols - 1) / cols, heads, n_seqs);
+  const int unit = dtype == CWM_BF16 ? 8 : 4;
+  const bool vec = N % unit == 0 && P % unit == 0 && xbc_ld % unit == 0 && ((uintptr_t)xbc % 16) == 0 && 16 * row / unit <= SCAN_PFV * 256;
+#define CWM_SCAN(T, VEC) \
+  launch_scan<T, VEC>(grid, split, stream, xbc, xbc_ld, dt_raw, dt_ld, dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, n_slots)
+  if (dtype == CWM_BF16) {
+    if (vec) CWM_SCAN(bf16_t, true); else CWM_SCAN(bf16_t, false);
+  } else if (dtype == CWM_F32) {
+    if (vec) CWM_SCAN(float, true); else CWM_SCAN(float, false);
+  } else {
     return cwm_fail("selective_scan: unknown dtype %d", dtype);
+  }
+#undef CWM_SCAN
   return cwm_launch_status("selective_scan");
 }

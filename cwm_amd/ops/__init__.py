@@ -1201,7 +1201,8 @@ def measure_mfma_rate(device: torch.device, blocks: int, rounds: int, launches: 
 # --------------------------------------------------------------------------- #
 # entry points that live in modules of their own; parts reach them as `ops.<name>` like the ones above
 from .sequence import (  # noqa: E402
-    MAX_CONV_TAPS, MAX_SSM_STATE, add_rows, cast_rows, causal_conv_silu, group_rmsnorm, selective_scan, sigmoid_mul, token_shift,
+    MAX_CONV_TAPS, MAX_SSM_STATE, add_rows, cast_rows, causal_conv_silu, group_rmsnorm, scan_state_elems, scan_state_pack,
+    scan_state_unpack, selective_scan, sigmoid_mul, token_shift,
 )
 from .routed import (  # noqa: E402
     MAX_EXPERTS, MAX_ROUTE_TOP, ExpertGroups, absorb_queries, combine_routed, expand_values, group_by_expert, grouped_gate_up,

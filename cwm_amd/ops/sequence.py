@@ -191,13 +191,47 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, 
     return out
 
 
+SCAN_ROWS = 16  # csrc/state_space.hip: rows of a head's state that one thread holds
+
+
+def scan_split(n_state: int) -> int:
+    """Lanes that share a column of a head's state (csrc/state_space.hip: cwm_scan_split)."""
+    split = 1
+    while split * SCAN_ROWS < n_state:
+        split *= 2
+    return split
+
+
+def scan_state_elems(heads: int, head_dim: int, n_state: int) -> int:
+    """float32 values that the scan kernel keeps for one request: every head's state padded to 16 * split rows."""
+    return heads * SCAN_ROWS * scan_split(n_state) * head_dim
+
+
+def scan_state_pack(states: torch.Tensor) -> torch.Tensor:
+    """[heads, n_state, head_dim] -> the flat order in which the scan kernel keeps it: per head [q][p][s][j] for row
+    4 (s + q split) + j of column p, rows from n_state on zero.  (For tests and for looking at a state.)"""
+    heads, n_state, head_dim = states.shape
+    split = scan_split(n_state)
+    padded = torch.zeros((heads, SCAN_ROWS * split, head_dim), dtype=states.dtype, device=states.device)
+    padded[:, :n_state] = states
+    # row n = 4 (s + q split) + j  ->  [q][s][j]
+    return padded.reshape(heads, SCAN_ROWS // 4, split, 4, head_dim).permute(0, 1, 4, 2, 3).reshape(-1).contiguous()
+
+
+def scan_state_unpack(flat: torch.Tensor, heads: int, head_dim: int, n_state: int) -> torch.Tensor:
+    """The inverse of `scan_state_pack`: [heads, n_state, head_dim]."""
+    split = scan_split(n_state)
+    rows = flat[: scan_state_elems(heads, head_dim, n_state)].reshape(heads, SCAN_ROWS // 4, head_dim, split, 4)
+    return rows.permute(0, 1, 3, 4, 2).reshape(heads, SCAN_ROWS * split, head_dim)[:, :n_state].contiguous()
+
+
 def selective_scan(
     xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, batch: Any,
     heads: int, head_dim: int, n_state: int, groups: int,
 ) -> torch.Tensor:
     """The recurrence S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x per head over each sequence of the step,
-    in float32, from and into the sequences' rows of `state` (float32 [slots, n], S of all heads first, each
-    [n_state, head_dim]).  `xbc` [T, heads * head_dim + 2 * groups * n_state] = [x | B | C]; `dt` [T, heads] before
+    in float32, from and into the sequences' rows of `state` (float32 [slots, n], n a multiple of 4; S of all heads
+    first, `scan_state_elems` values in the kernel's own order, see `scan_state_pack`).  `xbc` [T, heads * head_dim + 2 * groups * n_state] = [x | B | C]; `dt` [T, heads] before
     bias and softplus (rows may lie apart); `dt_bias`, `a_log`, `d_skip` float32 [heads].  Returns y float32
     [T, heads * head_dim]."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
@@ -211,8 +245,11 @@ def selective_scan(
     for name, t in (("dt_bias", dt_bias), ("A_log", a_log), ("D", d_skip)):
         if t.dtype != torch.float32 or t.shape != (heads,) or not t.is_contiguous():
             raise KernelError(f"{name} must be float32 [{heads}]")
-    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or state.shape[1] < heads * n_state * head_dim:
-        raise KernelError("the state must be a contiguous float32 [slots, n] tensor that holds every head's state")
+    if (
+        state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or state.shape[1] % 4 != 0
+        or state.shape[1] < scan_state_elems(heads, head_dim, n_state)
+    ):
+        raise KernelError("the state must be a contiguous float32 [slots, n] tensor, n a multiple of 4, that holds every head's state")
     if n_state > MAX_SSM_STATE:
         raise KernelError(f"a state of {n_state} rows is more than the {MAX_SSM_STATE} the scan kernel takes")
     if n_tokens != batch.n_tokens:

@@ -20,8 +20,8 @@ class SelectiveStateSpace(Mixer):
     then out = W_o norm(y * silu(z)) with a group norm of `norm_groups` parts.  The recurrence, its step sizes
     and decays and the gated norm run in float32 whatever the activation type.
 
-    A request's state is one float32 row: S of every head, then the last taps - 1 inputs of the convolution
-    (oldest first), so a portion of a prompt goes on exactly where the step before stopped."""
+    A request's state is one float32 row: S of every head (in the order the scan kernel holds it), then the last
+    taps - 1 inputs of the convolution (oldest first), so a portion of a prompt goes on where the step before stopped."""
 
     replayable = True
 
@@ -36,8 +36,8 @@ class SelectiveStateSpace(Mixer):
         self.inner = heads * head_dim
         self.channels = self.inner + 2 * groups * state  # what the convolution sees
         self.norm = PartChoice("group_rmsnorm", {"dim": self.inner, "eps": eps, "groups": norm_groups, "tensor": "norm"}).build("norm")
-        self.ssm_elems = heads * state * head_dim
-        self.state_elems = self.ssm_elems + (taps - 1) * self.channels
+        self.ssm_elems = ops.scan_state_elems(heads, head_dim, state)  # in the scan kernel's own order and padding
+        self.state_elems = -(-(self.ssm_elems + (taps - 1) * self.channels) // 4) * 4
 
     def cache_spec(self) -> StateSpec:
         return StateSpec((self.state_elems,), torch.float32)

@@ -116,32 +116,38 @@ def test_selective_scan_batch_and_portions(dtype, heads, head_dim, n_state, grou
     from cwm_amd import ops
 
     torch.manual_seed(heads * 7 + n_state)
-    inner, width = heads * head_dim, heads * head_dim + 2 * groups * n_state
+    inner, width = heads * head_dim, heads * head_dim + 2 * groups * n_state  # noqa: F841
     q_lens, starts, slots = [5, 1, 12], [0, 3, 40], [2, 0, 1]
     n = sum(q_lens)
     xbc = torch.randn(n, width).to(dtype)
     dt = (torch.randn(n, heads) - 1).to(dtype)
     dt_bias, a_log, d_skip = torch.randn(heads) * 0.5, torch.randn(heads) * 0.5, torch.randn(heads)
-    state = torch.randn(3, heads * n_state * head_dim + 11)
-    state[2, : heads * n_state * head_dim] = 0  # the sequence that starts
-    sd = state.to(DEV)
+    elems = heads * n_state * head_dim
+    state = torch.randn(3, elems + 11)
+    state[2, :elems] = 0  # the sequence that starts
+    # the kernel keeps a head's state in an order and padding of its own
+    n_dev = -(-(ops.scan_state_elems(heads, head_dim, n_state) + 11) // 4) * 4
+    pack = lambda rows: torch.stack([ops.scan_state_pack(r[:elems].reshape(heads, n_state, head_dim)) for r in rows])  # noqa: E731
+    sd = torch.full((3, n_dev), 5.0)
+    sd[:, : ops.scan_state_elems(heads, head_dim, n_state)] = pack(state)
+    sd = sd.to(DEV)
     gb, cb = _both(q_lens, starts, slots)
     wide = torch.zeros(n, width + heads + 6, dtype=dtype, device=DEV)
     wide[:, :width], wide[:, width : width + heads] = xbc.to(DEV), dt.to(DEV)
-    got = ops.selective_scan(wide[:, :width], wide[:, width : width + heads], dt_bias.to(DEV), a_log.to(DEV), d_skip.to(DEV), sd, gb, heads, head_dim, n_state, groups)
+    args = (dt_bias.to(DEV), a_log.to(DEV), d_skip.to(DEV))
+    got = ops.selective_scan(wide[:, :width], wide[:, width : width + heads], *args, sd, gb, heads, head_dim, n_state, groups)
     want = cpu_ops.selective_scan(xbc.float(), dt.float(), dt_bias, a_log, d_skip, state, cb, heads, head_dim, n_state, groups)
     tol = dict(rtol=2e-4, atol=2e-4)
     torch.testing.assert_close(got.cpu(), want, **tol)
-    torch.testing.assert_close(sd.cpu(), state, **tol)
-    # the same tokens one by one give the same bits as the portion did
-    sd2 = state.clone()
-    sd2[2, : heads * n_state * head_dim] = 0
-    # (restart the first sequence from zero and feed its five tokens singly)
-    sd2 = sd2.to(DEV)
+    for slot in range(3):
+        torch.testing.assert_close(ops.scan_state_unpack(sd[slot].cpu(), heads, head_dim, n_state).reshape(-1), state[slot, :elems], **tol)
+    assert torch.all(sd[:, ops.scan_state_elems(heads, head_dim, n_state) :] == 5.0)  # what lies behind the heads' states is not touched
+    # the same tokens one by one give the same bits as the portion did (the first sequence again, from zero)
+    sd2 = torch.zeros((3, n_dev), device=DEV)
     singles = []
     for i in range(5):
         one = _batch([1], [i], [2], DEV)
-        singles.append(ops.selective_scan(wide[i : i + 1, :width], wide[i : i + 1, width : width + heads], dt_bias.to(DEV), a_log.to(DEV), d_skip.to(DEV), sd2, one, heads, head_dim, n_state, groups))
+        singles.append(ops.selective_scan(wide[i : i + 1, :width], wide[i : i + 1, width : width + heads], *args, sd2, one, heads, head_dim, n_state, groups))
     assert torch.equal(torch.cat(singles), got[:5])
 
 
