@@ -127,16 +127,31 @@ extern "C" int cwm_conv_silu(const void* in, long in_ld, int dtype, const float*
 // of the values in 16 bytes, so a chunk is fetched in pieces of 16 bytes; otherwise value by value.
 #define SCAN_PFV 6  // most 16-byte pieces of a chunk that one thread fetches
 
-template <typename T, int THREADS, int TC, bool VEC>
+//
+// Long portions are cut into segments that run side by side (PHASE 1 and 2; PHASE 0 is the walk of whole portions):
+// `segments` holds, for every block z, {sequence, first token, end token, number j of the segment in its sequence,
+// the sequence's first entry in the scratch lists, segments of the sequence}.  PHASE 1: segment j < last walks its
+// tokens from a zero state and leaves that state and the product of its decays in entry 1 + j; the last segment's
+// block copies the sequence's state into entry 0.  PHASE 2: segment j starts from entry 0 carried through the
+// entries 1 .. j (S <- decay_i S + state_i), walks its tokens and writes y; the last one leaves the sequence's state.
+// No block reads a state that another block of the same launch writes.
+template <typename T, int THREADS, int TC, bool VEC, int PHASE>
 __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt_raw,
                                                                  long dt_ld, const float* __restrict__ dt_bias,
                                                                  const float* __restrict__ a_log, const float* __restrict__ d_skip,
                                                                  float* state, long state_ld, const int* __restrict__ slots,
                                                                  const int* __restrict__ cu_q, float* __restrict__ y, int heads, int P,
-                                                                 int N, int groups, int split, int n_slots) {
+                                                                 int N, int groups, int split, int n_slots,
+                                                                 const int* __restrict__ segments, float* seg_state, float* seg_decay) {
   extern __shared__ float lds[];
   const int h = blockIdx.y;
-  const int b = blockIdx.z;
+  int b = blockIdx.z, t0, t1, seg = 0, seg_base = 0, n_segs = 1;
+  if (PHASE == 0) {
+    t0 = cu_q[b], t1 = cu_q[b + 1];
+  } else {
+    const int* entry = segments + 6 * blockIdx.z;
+    b = entry[0], t0 = entry[1], t1 = entry[2], seg = entry[3], seg_base = entry[4], n_segs = entry[5];
+  }
   const int cols = THREADS / split;
   const int s = threadIdx.x % split;
   const int col = threadIdx.x / split;
@@ -154,16 +169,50 @@ __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __rest
   // thread's four rows are 16 bytes and the split lanes of a column lie side by side (rows from N on stay zero).
   float* st = (slot >= 0 && slot < n_slots) ? state + (size_t)slot * state_ld + (size_t)h * SCAN_ROWS * split * P : nullptr;
   float S[SCAN_ROWS];
+  const size_t head_elems = (size_t)SCAN_ROWS * split * P;
+  auto load_state = [&](const float* from) {  // null: zeros
 #pragma unroll
-  for (int q = 0; q < SCAN_ROWS / 4; ++q) {
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (st && live) v = *(const float4*)(st + (((size_t)q * P + p) * split + s) * 4);
-    S[4 * q + 0] = v.x, S[4 * q + 1] = v.y, S[4 * q + 2] = v.z, S[4 * q + 3] = v.w;
+    for (int q = 0; q < SCAN_ROWS / 4; ++q) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (from && live) v = *(const float4*)(from + (((size_t)q * P + p) * split + s) * 4);
+      S[4 * q + 0] = v.x, S[4 * q + 1] = v.y, S[4 * q + 2] = v.z, S[4 * q + 3] = v.w;
+    }
+  };
+  auto store_state = [&](float* to) {
+    if (to && live) {
+#pragma unroll
+      for (int q = 0; q < SCAN_ROWS / 4; ++q)
+        *(float4*)(to + (((size_t)q * P + p) * split + s) * 4) = make_float4(S[4 * q + 0], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
+    }
+  };
+  auto entry_state = [&](int k) { return seg_state + ((size_t)(seg_base + k) * heads + h) * head_elems; };
+  if (PHASE == 0) {
+    load_state(st);
+  } else if (PHASE == 1) {
+    if (seg == n_segs - 1) {  // the whole block: the sequence's state as it is, for the segments of the next launch
+      load_state(st);
+      store_state(entry_state(0));
+      return;
+    }
+    load_state(nullptr);
+  } else {
+    load_state(entry_state(0));
+    for (int i = 0; i < seg; ++i) {
+      const float d = seg_decay[(size_t)(seg_base + 1 + i) * heads + h];
+      const float* local = entry_state(1 + i);
+#pragma unroll
+      for (int q = 0; q < SCAN_ROWS / 4; ++q) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) v = *(const float4*)(local + (((size_t)q * P + p) * split + s) * 4);
+        S[4 * q + 0] = d * S[4 * q + 0] + v.x, S[4 * q + 1] = d * S[4 * q + 1] + v.y;
+        S[4 * q + 2] = d * S[4 * q + 2] + v.z, S[4 * q + 3] = d * S[4 * q + 3] + v.w;
+      }
+    }
   }
   const float bias = dt_bias[h];
   const float rate = -expf(a_log[h]);
   const float skip = d_skip[h];
-  const int t0 = cu_q[b], t1 = cu_q[b + 1];
+  float decays = 1.f;  // PHASE 1: the product of the segment's decays
 
   constexpr int U = 16 / sizeof(T);  // values in 16 bytes
   float pf[VEC ? 1 : SCAN_PF];
@@ -268,6 +317,7 @@ __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __rest
       if (FULL || tc < n_here) {
         const float* tok = lds + tc * row;
         const float a = av[tc];
+        if (PHASE == 1) decays *= a;
         const float x = tok[2 * NB + col];
         const float dx = dtv[tc] * x;
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -288,6 +338,7 @@ __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __rest
         xs[tc] = x;
       }
     }
+    if (PHASE == 1) return;  // only the state is wanted
     for (int off = 1; off < split; off <<= 1) {
 #pragma unroll
       for (int tc = 0; tc < TC; ++tc)
@@ -317,28 +368,41 @@ __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __rest
       __syncthreads();
     }
   }
-  if (st && live) {
-#pragma unroll
-    for (int q = 0; q < SCAN_ROWS / 4; ++q)
-      *(float4*)(st + (((size_t)q * P + p) * split + s) * 4) = make_float4(S[4 * q + 0], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
+  if (PHASE == 0) {
+    store_state(st);
+  } else if (PHASE == 1) {
+    store_state(entry_state(1 + seg));
+    if (threadIdx.x == 0) seg_decay[(size_t)(seg_base + 1 + seg) * heads + h] = decays;
+  } else if (seg == n_segs - 1) {
+    store_state(st);
   }
 }
 
 template <typename T, bool VEC>
 static void launch_scan(dim3 grid, int split, hipStream_t stream, const void* xbc, long xbc_ld, const void* dt_raw, long dt_ld,
                         const float* dt_bias, const float* a_log, const float* d_skip, float* state, long state_ld, const int* slots,
-                        const int* cu_q, float* y, int heads, int P, int N, int groups, int n_slots) {
+                        const int* cu_q, float* y, int heads, int P, int N, int groups, int n_slots, const int* segments, float* seg_state,
+                        float* seg_decay) {
   constexpr int THREADS = 256, TC = 16;
   const int row = 2 * SCAN_ROWS * split + THREADS / split;
   const size_t lds_bytes = (size_t)(TC * row + 2 * TC) * sizeof(float);
-  hipLaunchKernelGGL((selective_scan_kernel<T, THREADS, TC, VEC>), grid, dim3(THREADS), lds_bytes, stream, (const T*)xbc, xbc_ld,
-                     (const T*)dt_raw, dt_ld, dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots);
+#define CWM_SCAN_PHASE(PHASE)                                                                                                              \
+  hipLaunchKernelGGL((selective_scan_kernel<T, THREADS, TC, VEC, PHASE>), grid, dim3(THREADS), lds_bytes, stream, (const T*)xbc, xbc_ld,     \
+                     (const T*)dt_raw, dt_ld, dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, split, n_slots, \
+                     segments, seg_state, seg_decay)
+  if (!segments) {
+    CWM_SCAN_PHASE(0);
+  } else {
+    CWM_SCAN_PHASE(1);
+    CWM_SCAN_PHASE(2);
+  }
+#undef CWM_SCAN_PHASE
 }
 
 extern "C" int cwm_selective_scan(const void* xbc, long xbc_ld, const void* dt_raw, long dt_ld, int dtype, const float* dt_bias,
                                   const float* a_log, const float* d_skip, float* state, long state_ld, const int* slots,
                                   const int* cu_q, float* y, int n_tokens, int n_seqs, int heads, int P, int N, int groups, int n_slots,
-                                  hipStream_t stream) {
+                                  const int* segments, int n_segments, float* seg_state, float* seg_decay, hipStream_t stream) {
   CWM_REQUIRE(xbc && dt_raw && dt_bias && a_log && d_skip && state && slots && cu_q && y, "selective_scan: arguments missing");
   CWM_REQUIRE(heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0, "selective_scan: bad sizes");
   CWM_REQUIRE(N <= SCAN_ROWS * 16, "selective_scan: a state of %d rows, the kernel takes up to %d", N, SCAN_ROWS * 16);
@@ -351,11 +415,15 @@ extern "C" int cwm_selective_scan(const void* xbc, long xbc_ld, const void* dt_r
   const int cols = 256 / split;
   const int row = 2 * SCAN_ROWS * split + cols;
   CWM_REQUIRE(16 * row <= SCAN_PF * 256, "selective_scan: a chunk of tokens does not fit the threads' registers");
-  dim3 grid((P + cols - 1) / cols, heads, n_seqs);
+  // with a list of segments (6 numbers each; its scratch lists have an entry for every segment) the blocks' z counts those
+  CWM_REQUIRE(!segments || (n_segments > 0 && n_segments <= 65535 && seg_state && seg_decay && ((uintptr_t)seg_state % 16) == 0),
+              "selective_scan: a list of segments needs its scratch lists and at most 65535 entries");
+  dim3 grid((P + cols - 1) / cols, heads, segments ? n_segments : n_seqs);
   const int unit = dtype == CWM_BF16 ? 8 : 4;
   const bool vec = N % unit == 0 && P % unit == 0 && xbc_ld % unit == 0 && ((uintptr_t)xbc % 16) == 0 && 16 * row / unit <= SCAN_PFV * 256;
 #define CWM_SCAN(T, VEC) \
-  launch_scan<T, VEC>(grid, split, stream, xbc, xbc_ld, dt_raw, dt_ld, dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, n_slots)
+  launch_scan<T, VEC>(grid, split, stream, xbc, xbc_ld, dt_raw, dt_ld, dt_bias, a_log, d_skip, state, state_ld, slots, cu_q, y, heads, P, N, groups, n_slots, \
+                      segments, seg_state, seg_decay)
   if (dtype == CWM_BF16) {
     if (vec) CWM_SCAN(bf16_t, true); else CWM_SCAN(bf16_t, false);
   } else if (dtype == CWM_F32) {

@@ -225,6 +225,33 @@ def scan_state_unpack(flat: torch.Tensor, heads: int, head_dim: int, n_state: in
     return rows.permute(0, 1, 3, 4, 2).reshape(heads, SCAN_ROWS * split, head_dim)[:, :n_state].contiguous()
 
 
+SCAN_SEGMENT = 256  # tokens of a segment; a step with a longer portion runs its portions' segments side by side
+
+
+def _scan_segments(batch: Any, device: torch.device):
+    """The step's list of segments for the scan kernel (int32 [n, 6] on the device: sequence, first token, end token,
+    number of the segment in its sequence, the sequence's first scratch entry, segments of the sequence), or None if
+    no portion is longer than a segment.  Built once a step from the host's copy of the portions' lengths."""
+    q_lens = getattr(batch, "q_lens", None)
+    if not q_lens or max(q_lens) <= SCAN_SEGMENT:
+        return None
+    scratch = getattr(batch, "scratch", None)
+    if scratch is not None and "scan_segments" in scratch:
+        return scratch["scan_segments"]
+    rows, first, base = [], 0, 0
+    for b, q in enumerate(q_lens):
+        n = -(-q // SCAN_SEGMENT)
+        for j in range(n):
+            rows.append((b, first + j * SCAN_SEGMENT, first + min(q, (j + 1) * SCAN_SEGMENT), j, base, n))
+        first += q
+        base += n
+    host = torch.tensor(rows, dtype=torch.int32)
+    table = (host.pin_memory() if device.type == "cuda" else host).to(device, non_blocking=True)
+    if scratch is not None:
+        scratch["scan_segments"] = table
+    return table
+
+
 def selective_scan(
     xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, batch: Any,
     heads: int, head_dim: int, n_state: int, groups: int,
@@ -233,7 +260,9 @@ def selective_scan(
     in float32, from and into the sequences' rows of `state` (float32 [slots, n], n a multiple of 4; S of all heads
     first, `scan_state_elems` values in the kernel's own order, see `scan_state_pack`).  `xbc` [T, heads * head_dim + 2 * groups * n_state] = [x | B | C]; `dt` [T, heads] before
     bias and softplus (rows may lie apart); `dt_bias`, `a_log`, `d_skip` float32 [heads].  Returns y float32
-    [T, heads * head_dim]."""
+    [T, heads * head_dim].  Portions of up to `SCAN_SEGMENT` tokens are walked token by token, which gives the same
+    bits however a sequence is cut; a step with a longer portion (`batch.q_lens`) cuts its portions into segments that
+    run side by side and carries the state across them, which differs from the walk by rounding."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
     _need_gpu(xbc, dt, dt_bias, a_log, d_skip, state)
     _rows_2d(xbc, "xbc")
@@ -255,6 +284,14 @@ def selective_scan(
     if n_tokens != batch.n_tokens:
         raise KernelError("one row per token of the step is needed")
     y = torch.empty((n_tokens, inner), dtype=torch.float32, device=xbc.device)
+    segments = _scan_segments(batch, xbc.device)
+    seg_state = seg_decay = None
+    if segments is not None:
+        if segments.shape[0] > 65535:
+            segments = None  # (more segments than one launch counts: the portions are walked whole)
+        else:
+            seg_state = torch.empty((segments.shape[0], scan_state_elems(heads, head_dim, n_state)), dtype=torch.float32, device=xbc.device)
+            seg_decay = torch.empty((segments.shape[0], heads), dtype=torch.float32, device=xbc.device)
     lib = _build.load("state_space")
     _check(
         lib,
@@ -262,7 +299,8 @@ def selective_scan(
             _ptr(xbc), ctypes.c_long(xbc.stride(0) if n_tokens > 1 else xbc.shape[1]), _ptr(dt), ctypes.c_long(dt.stride(0) if n_tokens > 1 else heads),
             ctypes.c_int(_code(xbc.dtype)), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state), ctypes.c_long(state.shape[1]),
             _ptr(batch.state_slots), _ptr(batch.cu_q), _ptr(y), ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs), ctypes.c_int(heads),
-            ctypes.c_int(head_dim), ctypes.c_int(n_state), ctypes.c_int(groups), ctypes.c_int(state.shape[0]), _stream(),
+            ctypes.c_int(head_dim), ctypes.c_int(n_state), ctypes.c_int(groups), ctypes.c_int(state.shape[0]),
+            _ptr(segments), ctypes.c_int(segments.shape[0] if segments is not None else 0), _ptr(seg_state), _ptr(seg_decay), _stream(),
         ),
     )
     return y

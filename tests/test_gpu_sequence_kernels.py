@@ -22,7 +22,8 @@ def _batch(q_lens, starts, slots, device):
     seq = [b for b, q in enumerate(q_lens) for _ in range(q)]
     pos = [s + i for s, q in zip(starts, q_lens) for i in range(q)]
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)  # noqa: E731
-    return SimpleNamespace(n_tokens=cu[-1], n_seqs=len(q_lens), cu_q=i32(cu), seq_of_token=i32(seq), positions=i32(pos), state_slots=i32(slots))
+    return SimpleNamespace(n_tokens=cu[-1], n_seqs=len(q_lens), cu_q=i32(cu), seq_of_token=i32(seq), positions=i32(pos), state_slots=i32(slots),
+                           q_lens=list(q_lens), scratch={})
 
 
 def _both(q_lens, starts, slots):
@@ -149,6 +150,35 @@ def test_selective_scan_batch_and_portions(dtype, heads, head_dim, n_state, grou
         one = _batch([1], [i], [2], DEV)
         singles.append(ops.selective_scan(wide[i : i + 1, :width], wide[i : i + 1, width : width + heads], *args, sd2, one, heads, head_dim, n_state, groups))
     assert torch.equal(torch.cat(singles), got[:5])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,head_dim,n_state,groups", [(2, 16, 24, 1), (2, 64, 128, 2)])
+def test_selective_scan_long_portions_in_segments(dtype, heads, head_dim, n_state, groups):
+    """Portions longer than a segment run their segments side by side: a long fresh prompt, a decoded token and a
+    long portion that goes on from a state, in one step; the end states carry on into a second step."""
+    from cwm_amd import ops
+
+    torch.manual_seed(n_state)
+    inner, width = heads * head_dim, heads * head_dim + 2 * groups * n_state  # noqa: F841
+    elems, dev_elems = heads * n_state * head_dim, ops.scan_state_elems(heads, head_dim, n_state)
+    dt_bias, a_log, d_skip = torch.randn(heads) * 0.5 - 1, torch.rand(heads) * -3 - 1, torch.randn(heads)
+    args = (dt_bias.to(DEV), a_log.to(DEV), d_skip.to(DEV))
+    state = torch.randn(3, elems) * 0.3
+    state[0] = 0
+    sd = torch.stack([ops.scan_state_pack(r.reshape(heads, n_state, head_dim)) for r in state]).to(DEV)
+    assert sd.shape[1] == dev_elems
+    at = [0, 7, 100]
+    for q_lens in ([700, 1, 513], [1, 1, 300]):
+        n = sum(q_lens)
+        xbc, dt = (torch.randn(n, width) * 0.5).to(dtype), (torch.randn(n, heads) - 1).to(dtype)
+        gb, cb = _both(q_lens, at, [0, 1, 2])
+        got = ops.selective_scan(xbc.to(DEV), dt.to(DEV), *args, sd, gb, heads, head_dim, n_state, groups)
+        want = cpu_ops.selective_scan(xbc.float(), dt.float(), dt_bias, a_log, d_skip, state, cb, heads, head_dim, n_state, groups)
+        torch.testing.assert_close(got.cpu(), want, rtol=3e-4, atol=3e-4)
+        for slot in range(3):
+            torch.testing.assert_close(ops.scan_state_unpack(sd[slot].cpu(), heads, head_dim, n_state).reshape(-1), state[slot], rtol=3e-4, atol=3e-4)
+        at = [a + q for a, q in zip(at, q_lens)]
 
 
 def test_sigmoid_mul_and_cast():
