@@ -300,6 +300,97 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
   }
 }
 
+// Few rows an expert (a decode step): the product is bound by streaming the chosen experts' weights once.  A block
+// takes one row tile and 16 columns; its four wavefronts split K (wavefront w the steps w, w + 4, ...: together they
+// read whole lines of a weight row), each with STREAM_DEPTH steps of operands in flight while the ones before are
+// multiplied, and add their sums through LDS in the order of w.  Rows of a and W start at multiples of 16 bytes.
+#define STREAM_DEPTH 4
+
+template <typename T, bool GATED>
+__global__ void __launch_bounds__(256) grouped_stream_kernel(const T* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
+                                                             const T* __restrict__ w0, const T* __restrict__ w1, long w_stride,
+                                                             const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
+                                                             int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+  __shared__ float sums[4][GATED ? 2 : 1][64][4];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int tile = blockIdx.x;
+  int expert;
+  if (tile_expert) {
+    expert = tile < n_tiles ? tile_expert[tile] : -1;
+    if (expert < 0) return;
+  } else {
+    expert = blockIdx.z;
+  }
+  const int n0 = blockIdx.y * 16;
+  const int col = n0 + r;
+  const size_t at = (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K;
+  const T* wrow0 = w0 + at;
+  const T* wrow1 = GATED ? w1 + at : nullptr;
+  const int row = tile * TILE_ROWS + r;
+  long src = row_token ? row_token[row] : (row < n_rows ? row : -1);
+  const T* arow = src >= 0 ? a + (size_t)blockIdx.z * a_batch + (size_t)src * a_ld : nullptr;
+  constexpr int STEP = Frag<T>::K_STEP, PIECE = Frag<T>::PER_LANE;
+  const int steps = (K + STEP - 1) / STEP;
+  float4v acc0 = (float4v){0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
+  auto load_group = [&](Frag<T> (&fw0)[STREAM_DEPTH], Frag<T> (&fw1)[STREAM_DEPTH], Frag<T> (&fa)[STREAM_DEPTH], int first) {
+#pragma unroll
+    for (int d = 0; d < STREAM_DEPTH; ++d) {
+      const int step = wave + 4 * (first + d);
+      const int k = step * STEP + j * PIECE;
+      if (step < steps && k < K) {
+        fw0[d].load16(wrow0 + k);
+        if (GATED) fw1[d].load16(wrow1 + k);
+        if (arow) fa[d].load16(arow + k); else fa[d].zero();
+      } else {
+        fw0[d].zero();
+        if (GATED) fw1[d].zero();
+        fa[d].zero();
+      }
+    }
+  };
+  auto multiply_group = [&](const Frag<T> (&fw0)[STREAM_DEPTH], const Frag<T> (&fw1)[STREAM_DEPTH], const Frag<T> (&fa)[STREAM_DEPTH]) {
+#pragma unroll
+    for (int d = 0; d < STREAM_DEPTH; ++d) {
+      acc0 = Frag<T>::mma(fw0[d], fa[d], acc0);
+      if (GATED) acc1 = Frag<T>::mma(fw1[d], fa[d], acc1);
+    }
+  };
+  Frag<T> w0a[STREAM_DEPTH], w1a[STREAM_DEPTH], ra[STREAM_DEPTH], w0b[STREAM_DEPTH], w1b[STREAM_DEPTH], rb[STREAM_DEPTH];
+  const int groups = (steps + 4 * STREAM_DEPTH - 1) / (4 * STREAM_DEPTH);  // of STREAM_DEPTH steps a wavefront
+  load_group(w0a, w1a, ra, 0);
+  for (int g = 0; g < groups; g += 2) {
+    load_group(w0b, w1b, rb, (g + 1) * STREAM_DEPTH);  // beyond K: zeros
+    multiply_group(w0a, w1a, ra);
+    load_group(w0a, w1a, ra, (g + 2) * STREAM_DEPTH);
+    multiply_group(w0b, w1b, rb);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    sums[wave][0][lane][i] = acc0[i];
+    if (GATED) sums[wave][GATED ? 1 : 0][lane][i] = acc1[i];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  if (!tile_expert && row >= n_rows) return;
+  const size_t base = (size_t)blockIdx.z * out_batch + (size_t)row * out_ld;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = n0 + 4 * j + i;
+    if (c >= N) continue;
+    float v = ((sums[0][0][lane][i] + sums[1][0][lane][i]) + sums[2][0][lane][i]) + sums[3][0][lane][i];
+    if (GATED) {
+      const float u = ((sums[0][GATED ? 1 : 0][lane][i] + sums[1][GATED ? 1 : 0][lane][i]) + sums[2][GATED ? 1 : 0][lane][i]) + sums[3][GATED ? 1 : 0][lane][i];
+      v = v / (1.f + expf(-v)) * u;
+    }
+    if (out_dtype == CWM_F32)
+      ((float*)out)[base + c] = v;
+    else
+      ((bf16_t*)out)[base + c] = f32_to_bf16(v);
+  }
+}
+
 template <typename T, int RT, int CT, int WR, bool GATED>
 static void launch_grouped(bool vec, int tiles, int n_batch, hipStream_t stream, const T* a, long a_ld, long a_batch, const int* row_token,
                            const T* w0, const T* w1, long w_stride, const int* tile_expert, int n_tiles, void* out, int out_dtype,
@@ -349,6 +440,20 @@ extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int d
       else CWM_GROUPED(T, 1, 1, 1, false);                                      \
     }                                                                           \
   } while (0)
+  if (tiles_a_block == 1 && vec && (dtype == CWM_BF16 || dtype == CWM_F32)) {
+    // the weight-streaming shape
+    dim3 grid(tiles, (N + 15) / 16, nb);
+#define CWM_STREAMED(T, GATED)                                                                                                             \
+  hipLaunchKernelGGL((grouped_stream_kernel<T, GATED>), grid, dim3(256), 0, stream, (const T*)a, a_ld, a_batch, row_token, (const T*)w0,     \
+                     (const T*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K)
+    if (dtype == CWM_BF16) {
+      if (w1) CWM_STREAMED(bf16_t, true); else CWM_STREAMED(bf16_t, false);
+    } else {
+      if (w1) CWM_STREAMED(float, true); else CWM_STREAMED(float, false);
+    }
+#undef CWM_STREAMED
+    return cwm_launch_status("grouped_product");
+  }
   if (dtype == CWM_BF16)
     CWM_GROUPED_SHAPES(bf16_t);
   else if (dtype == CWM_F32)
