@@ -140,3 +140,22 @@ extern "C" int cwm_sigmoid_mul(const void* a, long a_ld, const void* g, long g_l
   hipLaunchKernelGGL(sigmoid_mul_kernel, dim3(n_rows, gy), dim3(256), 0, stream, a, a_ld, g, g_ld, out, out_ld, dtype, width);
   return cwm_launch_status("sigmoid_mul");
 }
+
+// out[r][0..width) = src[r][0..width) for rows of `src_ld` and `out_ld` elements of 2 or 4 bytes (columns of one
+// tensor into columns of another).
+template <typename T>
+__global__ void __launch_bounds__(256) copy_columns_kernel(const T* __restrict__ src, long src_ld, T* __restrict__ out, long out_ld, int width) {
+  const size_t r = blockIdx.x;
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x) out[r * out_ld + i] = src[r * src_ld + i];
+}
+
+extern "C" int cwm_copy_columns(const void* src, long src_ld, void* out, long out_ld, int dtype, long n_rows, int width, hipStream_t stream) {
+  CWM_REQUIRE(src && out && n_rows >= 0 && width > 0 && n_rows <= 2147483647L, "copy_columns: bad arguments");
+  if (n_rows == 0) return 0;
+  dim3 grid((unsigned)n_rows, (width + 1023) / 1024);
+  if (dtype == CWM_BF16)
+    hipLaunchKernelGGL(copy_columns_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)src, src_ld, (bf16_t*)out, out_ld, width);
+  else
+    hipLaunchKernelGGL(copy_columns_kernel<float>, grid, dim3(256), 0, stream, (const float*)src, src_ld, (float*)out, out_ld, width);
+  return cwm_launch_status("copy_columns");
+}

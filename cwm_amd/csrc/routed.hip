@@ -391,6 +391,155 @@ __global__ void __launch_bounds__(256) grouped_stream_kernel(const T* __restrict
   }
 }
 
+// Many rows an expert, bfloat16, K a multiple of 64: a block of four wavefronts (2 x 2) takes 8 row tiles of one expert
+// and 128 rows of weights (128 columns of the result; with two weights 64 columns of each), 64 values of k a step.
+// The step's 16 KB of rows and 16 KB of weights go from global memory to registers while the step before is
+// multiplied, then into the other of two LDS buffers (16-byte pieces, a row's pieces XOR-swizzled by the row so that
+// the lanes of a matrix operand read different banks); every wavefront multiplies 64 rows by 64 weight rows from there.
+template <bool GATED>
+__global__ void __launch_bounds__(256) grouped_tiled_kernel(const bf16_t* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
+                                                            const bf16_t* __restrict__ w0, const bf16_t* __restrict__ w1, long w_stride,
+                                                            const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
+                                                            int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+  extern __shared__ uint4 tiled_lds[];  // [2 buffers][rows: 128 x 8 pieces | weights: 128 x 8 pieces]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wr = wave >> 1, wc = wave & 1;
+  const int r = lane & 15, j = lane >> 4;
+  const int block_tile0 = blockIdx.x * 8;
+  int expert;
+  if (tile_expert) {
+    expert = block_tile0 < n_tiles ? tile_expert[block_tile0] : -1;
+    if (expert < 0) return;
+  } else {
+    expert = blockIdx.z;
+  }
+  constexpr int OUT_COLS = GATED ? 64 : 128;  // columns of the result a block makes
+  const int n0 = blockIdx.y * OUT_COLS;
+  // what this thread fetches every step: pieces id = threadIdx.x + 256 i, i < 4, of the rows and of the weights
+  const bf16_t* src_a[4];
+  const bf16_t* src_w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int id = threadIdx.x + 256 * i;
+    const int row = id >> 3, piece = id & 7;
+    const int tile = block_tile0 + (row >> 4);
+    const bool live = tile_expert ? (tile < n_tiles && tile_expert[tile] == expert) : tile * TILE_ROWS < n_rows;
+    const int list_row = tile * TILE_ROWS + (row & 15);
+    long src = -1;
+    if (live) src = row_token ? row_token[list_row] : (list_row < n_rows ? list_row : -1);
+    src_a[i] = src >= 0 ? a + (size_t)blockIdx.z * a_batch + (size_t)src * a_ld + piece * 8 : nullptr;
+    int col;  // the weight row: with two weights rows 0..63 are the first one's, 64..127 the second one's
+    const bf16_t* w = w0;
+    if (GATED) {
+      col = n0 + (row & 63);
+      if (row >= 64) w = w1;
+    } else {
+      col = n0 + row;
+    }
+    src_w[i] = w + (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K + piece * 8;
+  }
+  // two steps of operands on their way: what is fetched at the start of step k is put into LDS at the end of step k + 1
+  uint4 ra[2][4], rw[2][4];
+  auto fetch = [&](uint4 (&fa)[4], uint4 (&fw)[4], int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool inside = k0 < K;
+      fa[i] = (inside && src_a[i]) ? *(const uint4*)(src_a[i] + k0) : make_uint4(0, 0, 0, 0);
+      fw[i] = inside ? *(const uint4*)(src_w[i] + k0) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stage = [&](const uint4 (&fa)[4], const uint4 (&fw)[4], int buf) {
+    uint4* rows = tiled_lds + buf * 2048;
+    uint4* weights = rows + 1024;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int id = threadIdx.x + 256 * i;
+      const int row = id >> 3, piece = id & 7;
+      rows[row * 8 + (piece ^ (row & 7))] = fa[i];
+      weights[row * 8 + (piece ^ (row & 7))] = fw[i];
+    }
+  };
+  float4v acc0[4][GATED ? 2 : 4], acc1[4][GATED ? 2 : 1];
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+    for (int ct = 0; ct < (GATED ? 2 : 4); ++ct) acc0[rt][ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ct = 0; ct < (GATED ? 2 : 1); ++ct) acc1[rt][ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+  }
+  auto multiply = [&](int buf) {
+    const uint4* rows = tiled_lds + buf * 2048;
+    const uint4* weights = rows + 1024;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int piece = half * 4 + j;
+      Frag8 fa[4], fw[4];
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt) {
+        const int row = wr * 64 + rt * 16 + r;
+        fa[rt].u = rows[row * 8 + (piece ^ (row & 7))];
+      }
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        // weight rows of this wavefront: 64 in a row, or (two weights) 32 of each
+        const int row = GATED ? (ct < 2 ? wc * 32 + ct * 16 + r : 64 + wc * 32 + (ct - 2) * 16 + r) : wc * 64 + ct * 16 + r;
+        fw[ct].u = weights[row * 8 + (piece ^ (row & 7))];
+      }
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt) {
+        if (GATED) {
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) {
+            acc0[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[ct].v, fa[rt].v, acc0[rt][ct], 0, 0, 0);
+            acc1[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[2 + ct].v, fa[rt].v, acc1[rt][ct], 0, 0, 0);
+          }
+        } else {
+#pragma unroll
+          for (int ct = 0; ct < 4; ++ct) acc0[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[ct].v, fa[rt].v, acc0[rt][ct], 0, 0, 0);
+        }
+      }
+    }
+  };
+  fetch(ra[0], rw[0], 0);
+  stage(ra[0], rw[0], 0);
+  fetch(ra[0], rw[0], 64);  // for step 1, staged at the end of step 0
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += 128) {  // two steps a turn, so that the two register sets keep their names
+    fetch(ra[1], rw[1], k0 + 128);
+    multiply(0);
+    stage(ra[0], rw[0], 1);
+    __syncthreads();
+    if (k0 + 64 >= K) break;
+    fetch(ra[0], rw[0], k0 + 192);
+    multiply(1);
+    stage(ra[1], rw[1], 0);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt) {
+    const int tile = block_tile0 + wr * 4 + rt;
+    const bool live = tile_expert ? (tile < n_tiles && tile_expert[tile] == expert) : tile * TILE_ROWS < n_rows;
+    if (!live) continue;
+    const int row = tile * TILE_ROWS + r;
+    if (!tile_expert && row >= n_rows) continue;
+    const size_t base = (size_t)blockIdx.z * out_batch + (size_t)row * out_ld;
+#pragma unroll
+    for (int ct = 0; ct < (GATED ? 2 : 4); ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = n0 + (GATED ? wc * 32 : wc * 64) + ct * 16 + 4 * j + i;
+        if (c >= N) continue;
+        float v = acc0[rt][ct][i];
+        if (GATED) v = v / (1.f + expf(-v)) * acc1[rt][ct][i];
+        if (out_dtype == CWM_F32)
+          ((float*)out)[base + c] = v;
+        else
+          ((bf16_t*)out)[base + c] = f32_to_bf16(v);
+      }
+  }
+}
+
 template <typename T, int RT, int CT, int WR, bool GATED>
 static void launch_grouped(bool vec, int tiles, int n_batch, hipStream_t stream, const T* a, long a_ld, long a_batch, const int* row_token,
                            const T* w0, const T* w1, long w_stride, const int* tile_expert, int n_tiles, void* out, int out_dtype,
@@ -452,6 +601,18 @@ extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int d
       if (w1) CWM_STREAMED(float, true); else CWM_STREAMED(float, false);
     }
 #undef CWM_STREAMED
+    return cwm_launch_status("grouped_product");
+  }
+  if (tiles_a_block == 8 && vec && dtype == CWM_BF16 && K % 64 == 0) {
+    // the shape that goes through LDS
+    const size_t lds_bytes = 2 * 2048 * sizeof(uint4);
+    dim3 grid((tiles + 7) / 8, w1 ? (N + 63) / 64 : (N + 127) / 128, nb);
+    if (w1)
+      hipLaunchKernelGGL(grouped_tiled_kernel<true>, grid, dim3(256), lds_bytes, stream, (const bf16_t*)a, a_ld, a_batch, row_token,
+                         (const bf16_t*)w0, (const bf16_t*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+    else
+      hipLaunchKernelGGL(grouped_tiled_kernel<false>, grid, dim3(256), lds_bytes, stream, (const bf16_t*)a, a_ld, a_batch, row_token,
+                         (const bf16_t*)w0, (const bf16_t*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
     return cwm_launch_status("grouped_product");
   }
   if (dtype == CWM_BF16)

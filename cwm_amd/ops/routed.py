@@ -171,8 +171,17 @@ def absorb_queries(q: torch.Tensor, lead: int, weight: torch.Tensor) -> torch.Te
     n_tokens, heads, width = q.shape
     n = weight.shape[1]
     out = torch.empty((n_tokens, heads, lead + n), dtype=q.dtype, device=q.device)
-    if lead:
-        out[:, :, :lead].copy_(q[:, :, :lead])
+    if lead and n_tokens:
+        # the leading elements of every head as they are: rows of `width` into rows of `lead + n`, one a (token, head)
+        _, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+        lib = _build.load("groupnorm")
+        _check(
+            lib,
+            lib.cwm_copy_columns(
+                _ptr(q), ctypes.c_long(width), _ptr(out), ctypes.c_long(lead + n), ctypes.c_int(_code(q.dtype)),
+                ctypes.c_long(n_tokens * heads), ctypes.c_int(lead), _stream(),
+            ),
+        )
     if n_tokens:
         tiles = _tiles_a_block(n_tokens)
         _grouped(q.view(-1)[lead:], heads * width, width, None, weight, None, out.view(-1)[lead:], heads * (lead + n), lead + n, n_tokens, heads, tiles)

@@ -208,7 +208,7 @@ def test_route_top(n_experts, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n_tokens,dim,hidden,n_experts,top", [(1, 64, 32, 8, 4), (9, 192, 96, 8, 4), (200, 72, 40, 3, 2), (300, 64, 50, 4, 1), (33, 100, 36, 16, 3), (1200, 64, 48, 2, 1), (700, 40, 72, 3, 2)])
+@pytest.mark.parametrize("n_tokens,dim,hidden,n_experts,top", [(1, 64, 32, 8, 4), (9, 192, 96, 8, 4), (200, 72, 40, 3, 2), (300, 64, 50, 4, 1), (33, 100, 36, 16, 3), (1200, 64, 48, 2, 1), (700, 40, 72, 3, 2), (1300, 128, 64, 2, 2), (900, 192, 200, 3, 1)])
 def test_routed_experts_pipeline(dtype, n_tokens, dim, hidden, n_experts, top):
     """Grouping, both grouped products and the weighted sum, against one product per pair; sizes that are no
     multiple of a lane's piece take the kernels' element-wise loads."""
