@@ -157,10 +157,12 @@ class ShapeBench:
         embedding_only = model.tensor_names("embedding") - head_names  # tables of which a step reads one row a token
         # routed experts: a token is multiplied with `top` of a layer's `n_experts` expert matrices only
         routed = {}
+        self.expert_bytes = []  # per routed feed-forward: (bytes of all its experts, experts a token uses, experts)
         for layer, block in zip(model.plan.layers, model.blocks):
             for role, part in block.parts.items():
                 if hasattr(part, "n_experts") and hasattr(part, "top"):
                     routed[layer.prefix + block.names[role] + "e"] = part.top / part.n_experts
+                    self.expert_bytes.append([0, part.top, part.n_experts, layer.prefix + block.names[role] + "e"])
         for name, spec in model.tensor_specs().items():
             count = 1
             for n in spec.shape:
@@ -168,6 +170,9 @@ class ShapeBench:
             if name in embedding_only:
                 continue
             self.weight_bytes += count * self.esize
+            for entry in self.expert_bytes:
+                if name.startswith(entry[3]):
+                    entry[0] += count * self.esize
             if len(spec.shape) == 2:
                 if name in head_names:
                     self.head_params += count
@@ -194,8 +199,10 @@ class ShapeBench:
         return total
 
     def step_bytes(self, batch, ctx):
-        """What a decode step of `batch` requests at `ctx` tokens has to read: every weight once, and their cache."""
-        return self.weight_bytes + self.cache_bytes(batch, ctx)
+        """What a decode step of `batch` requests at `ctx` tokens has to read: every weight once (of routed experts
+        those that `batch` tokens with independent, even choices use: E (1 - (1 - top / E) ** batch) of E), and their cache."""
+        unused = sum(size * (1 - top / experts) ** batch for size, top, experts, _ in self.expert_bytes)
+        return self.weight_bytes - int(unused) + self.cache_bytes(batch, ctx)
 
     def prefill_flops(self, n_tokens, offset=0):
         """Flops of a portion of `n_tokens` after `offset` cached tokens whose last token's logits are wanted:
@@ -346,7 +353,8 @@ def compare_lapevik(args, device):
                 tok_s, ms = bench.decode_run(batch, args.context, args.steps, args.warmup)
                 row[label][f"decode_b{batch}_tok_s"] = round(tok_s, 1)
                 row[label][f"decode_b{batch}_ms"] = round(ms, 3)
-                row[label][f"decode_b{batch}_frac_of_all_weights"] = round(bench.step_bytes(batch, args.context) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+                row[label][f"decode_b{batch}_read_gb"] = round(bench.step_bytes(batch, args.context) / 1e9, 3)
+                row[label][f"decode_b{batch}_frac"] = round(bench.step_bytes(batch, args.context) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
             bench.close()
         out["sizes"][name] = row
     return out

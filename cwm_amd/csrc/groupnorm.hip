@@ -4,7 +4,8 @@
 //                 the row x = sum_p src[p][row] (* silu(gate[row]) if a gate is given), float32 arithmetic.
 //                 One entry point serves the norm of chosen rows into a fresh tensor, the norm of rows where they
 //                 lie (dst == src; the rows may be columns of a wider tensor) and the norm that adds into the
-//                 float32 residual stream (accumulate).
+//                 float32 residual stream (accumulate); the rows as they then stand can be left in a second tensor of
+//                 another type as well (the next sublayer's input).
 //   token shift   s_t = h_t + (h_(t-1) - h_t) * mu on the float32 stream, the previous token of a portion's first
 //                 token coming from the sequence's state, which receives the portion's last h.
 //   sigmoid gate  out = a * sigmoid(g).
@@ -34,7 +35,7 @@ __global__ void __launch_bounds__(256) group_norm_kernel(const void* src, int sr
                                                          long partial_stride, const void* gate, int gate_dtype,
                                                          long gate_ld, const void* __restrict__ weight, int w_dtype, void* dst,
                                                          int dst_dtype, long dst_ld, const int* __restrict__ rows, int part,
-                                                         float eps, int accumulate) {
+                                                         float eps, int accumulate, void* __restrict__ copy, int copy_dtype, long copy_ld) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int g = blockIdx.y;
@@ -67,13 +68,15 @@ __global__ void __launch_bounds__(256) group_norm_kernel(const void* src, int sr
     float y = v * inv * load_as_f32(weight, w_dtype, (size_t)g * part + i);
     if (accumulate) y += load_as_f32(dst, dst_dtype, d0 + i);
     store_from_f32(dst, dst_dtype, d0 + i, y);
+    if (copy) store_from_f32(copy, copy_dtype, (size_t)r * copy_ld + (size_t)g * part + i, y);  // what dst now holds, in another type
   }
 }
 
 // src: [n_partials][.][src_ld] (rows `rows[r]` or r), dst: [n_rows][dst_ld]; dim = groups * part elements of a row.
 extern "C" int cwm_group_norm(const void* src, int src_dtype, long src_ld, int n_partials, long partial_stride, const void* gate,
                               int gate_dtype, long gate_ld, const void* weight, int w_dtype, void* dst, int dst_dtype, long dst_ld,
-                              const int* rows, int n_rows, int dim, int groups, float eps, int accumulate, hipStream_t stream) {
+                              const int* rows, int n_rows, int dim, int groups, float eps, int accumulate, void* copy, int copy_dtype,
+                              long copy_ld, hipStream_t stream) {
   CWM_REQUIRE(src && weight && dst, "group_norm: arguments missing");
   CWM_REQUIRE(n_rows >= 0 && dim > 0 && groups > 0 && dim % groups == 0, "group_norm: %d elements do not divide into %d groups", dim, groups);
   CWM_REQUIRE(n_partials >= 1 && src_ld >= dim && dst_ld >= dim && (!gate || gate_ld >= dim), "group_norm: rows shorter than %d", dim);
@@ -81,7 +84,7 @@ extern "C" int cwm_group_norm(const void* src, int src_dtype, long src_ld, int n
   // a thread re-reads what it has not kept after it has written its own elements only: in place is safe
   if (n_rows == 0) return 0;
   hipLaunchKernelGGL(group_norm_kernel, dim3(n_rows, groups), dim3(256), 0, stream, src, src_dtype, src_ld, n_partials, partial_stride,
-                     gate, gate_dtype, gate_ld, weight, w_dtype, dst, dst_dtype, dst_ld, rows, dim / groups, eps, accumulate);
+                     gate, gate_dtype, gate_ld, weight, w_dtype, dst, dst_dtype, dst_ld, rows, dim / groups, eps, accumulate, copy, copy_dtype, copy_ld);
   return cwm_launch_status("group_norm");
 }
 

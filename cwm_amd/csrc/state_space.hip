@@ -325,14 +325,14 @@ __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __rest
         for (int q = 0; q < SCAN_ROWS / 4; ++q) {
           const float4 Bq = *(const float4*)(tok + 4 * (s + q * split));
           const float4 Cq = *(const float4*)(tok + NB + 4 * (s + q * split));
-          S[4 * q + 0] = a * S[4 * q + 0] + Bq.x * dx;
-          S[4 * q + 1] = a * S[4 * q + 1] + Bq.y * dx;
-          S[4 * q + 2] = a * S[4 * q + 2] + Bq.z * dx;
-          S[4 * q + 3] = a * S[4 * q + 3] + Bq.w * dx;
-          acc[0] += S[4 * q + 0] * Cq.x;
-          acc[1] += S[4 * q + 1] * Cq.y;
-          acc[2] += S[4 * q + 2] * Cq.z;
-          acc[3] += S[4 * q + 3] * Cq.w;
+          S[4 * q + 0] = fmaf(a, S[4 * q + 0], Bq.x * dx);
+          S[4 * q + 1] = fmaf(a, S[4 * q + 1], Bq.y * dx);
+          S[4 * q + 2] = fmaf(a, S[4 * q + 2], Bq.z * dx);
+          S[4 * q + 3] = fmaf(a, S[4 * q + 3], Bq.w * dx);
+          acc[0] = fmaf(S[4 * q + 0], Cq.x, acc[0]);
+          acc[1] = fmaf(S[4 * q + 1], Cq.y, acc[1]);
+          acc[2] = fmaf(S[4 * q + 2], Cq.z, acc[2]);
+          acc[3] = fmaf(S[4 * q + 3], Cq.w, acc[3]);
         }
         part[tc] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
         xs[tc] = x;
@@ -378,6 +378,63 @@ __global__ void __launch_bounds__(THREADS) selective_scan_kernel(const T* __rest
   }
 }
 
+// A step in which every sequence brings one token (decoding): no chunk, no LDS.  Thread (p, s) as above; its 16 values
+// of B and of C, x, dt and its 16 state values are all asked for at once, so the step waits for memory once.
+template <typename T>
+__global__ void __launch_bounds__(256) selective_scan_single_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt_raw,
+                                                                    long dt_ld, const float* __restrict__ dt_bias,
+                                                                    const float* __restrict__ a_log, const float* __restrict__ d_skip,
+                                                                    float* state, long state_ld, const int* __restrict__ slots,
+                                                                    float* __restrict__ y, int heads, int P, int N, int groups, int split,
+                                                                    int n_slots) {
+  const int h = blockIdx.y;
+  const int t = blockIdx.z;  // the sequence, and its one token
+  const int cols = 256 / split;
+  const int s = threadIdx.x % split;
+  const int p = blockIdx.x * cols + threadIdx.x / split;
+  const bool live = p < P;
+  const int pc = live ? p : P - 1;
+  const int g = h / (heads / groups);
+  const int inner = heads * P;
+  const int slot = slots[t];
+  float* st = (slot >= 0 && slot < n_slots) ? state + (size_t)slot * state_ld + (size_t)h * SCAN_ROWS * split * P : nullptr;
+  const T* row = xbc + (size_t)t * xbc_ld;
+  const T* Bt = row + inner + (size_t)g * N;
+  const T* Ct = Bt + (size_t)groups * N;
+  float S[SCAN_ROWS], Bv[SCAN_ROWS], Cv[SCAN_ROWS];
+#pragma unroll
+  for (int q = 0; q < SCAN_ROWS / 4; ++q) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (st && live) v = *(const float4*)(st + (((size_t)q * P + p) * split + s) * 4);
+    S[4 * q + 0] = v.x, S[4 * q + 1] = v.y, S[4 * q + 2] = v.z, S[4 * q + 3] = v.w;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int n = 4 * (s + q * split) + jj;
+      Bv[4 * q + jj] = n < N ? Elem<T>::load(Bt + n) : 0.f;
+      Cv[4 * q + jj] = n < N ? Elem<T>::load(Ct + n) : 0.f;
+    }
+  }
+  const float x = Elem<T>::load(row + (size_t)h * P + pc);
+  const float z = Elem<T>::load(dt_raw + (size_t)t * dt_ld + h) + dt_bias[h];
+  const float dt = z > 20.f ? z : log1pf(expf(z));
+  const float a = expf(-expf(a_log[h]) * dt);
+  const float dx = dt * x;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < SCAN_ROWS; ++i) {  // the same operations in the same order as the walk of a chunk
+    S[i] = fmaf(a, S[i], Bv[i] * dx);
+    acc[i & 3] = fmaf(S[i], Cv[i], acc[i & 3]);
+  }
+  float part = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+  for (int off = 1; off < split; off <<= 1) part += __shfl_xor(part, off, CWM_WAVE);
+  if (live && s == 0) y[(size_t)t * inner + (size_t)h * P + p] = part + d_skip[h] * x;
+  if (st && live) {
+#pragma unroll
+    for (int q = 0; q < SCAN_ROWS / 4; ++q)
+      *(float4*)(st + (((size_t)q * P + p) * split + s) * 4) = make_float4(S[4 * q + 0], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
+  }
+}
+
 template <typename T, bool VEC>
 static void launch_scan(dim3 grid, int split, hipStream_t stream, const void* xbc, long xbc_ld, const void* dt_raw, long dt_ld,
                         const float* dt_bias, const float* a_log, const float* d_skip, float* state, long state_ld, const int* slots,
@@ -419,6 +476,18 @@ extern "C" int cwm_selective_scan(const void* xbc, long xbc_ld, const void* dt_r
   CWM_REQUIRE(!segments || (n_segments > 0 && n_segments <= 65535 && seg_state && seg_decay && ((uintptr_t)seg_state % 16) == 0),
               "selective_scan: a list of segments needs its scratch lists and at most 65535 entries");
   dim3 grid((P + cols - 1) / cols, heads, segments ? n_segments : n_seqs);
+  if (!segments && n_tokens == n_seqs) {  // one token a sequence
+    dim3 single((P + cols - 1) / cols, heads, n_seqs);
+    if (dtype == CWM_BF16)
+      hipLaunchKernelGGL(selective_scan_single_kernel<bf16_t>, single, dim3(256), 0, stream, (const bf16_t*)xbc, xbc_ld, (const bf16_t*)dt_raw, dt_ld,
+                         dt_bias, a_log, d_skip, state, state_ld, slots, y, heads, P, N, groups, split, n_slots);
+    else if (dtype == CWM_F32)
+      hipLaunchKernelGGL(selective_scan_single_kernel<float>, single, dim3(256), 0, stream, (const float*)xbc, xbc_ld, (const float*)dt_raw, dt_ld,
+                         dt_bias, a_log, d_skip, state, state_ld, slots, y, heads, P, N, groups, split, n_slots);
+    else
+      return cwm_fail("selective_scan: unknown dtype %d", dtype);
+    return cwm_launch_status("selective_scan");
+  }
   const int unit = dtype == CWM_BF16 ? 8 : 4;
   const bool vec = N % unit == 0 && P % unit == 0 && xbc_ld % unit == 0 && ((uintptr_t)xbc % 16) == 0 && 16 * row / unit <= SCAN_PFV * 256;
 #define CWM_SCAN(T, VEC) \

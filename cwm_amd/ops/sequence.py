@@ -37,14 +37,15 @@ def group_rmsnorm(
     out: Optional[torch.Tensor] = None,
     accumulate: bool = False,
     gate: Optional[torch.Tensor] = None,
+    copy: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """weight * x_g / sqrt(mean(x_g^2) + eps) for each of `groups` equal consecutive parts x_g of every row, float32
     arithmetic.  `x` is [T, D] (rows may lie apart) or float32 partial sums [P, T, D], added in order first; with
     `gate` ([T, D]) the row is multiplied by silu(gate) before the norm.  `rows` (int32 [R]) chooses rows.  The
     result goes to a new [R, D] tensor of `out_dtype`, or into `out` ([R, D], which may be `x` itself), added to what
-    is there if `accumulate`."""
+    is there if `accumulate`.  `copy` (contiguous [R, D] of any type) also receives the rows as `out` then holds them."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
-    _need_gpu(x, weight, rows, out, gate)
+    _need_gpu(x, weight, rows, out, gate, copy)
     n_partials, partial_stride = 1, 0
     if x.dim() == 3:
         if x.dtype != torch.float32 or not x.is_contiguous():
@@ -76,6 +77,8 @@ def group_rmsnorm(
         if tuple(gate.shape) != (n_tokens, dim):
             raise KernelError(f"gate {tuple(gate.shape)} does not fit x")
         gate_ld = gate.stride(0) if n_tokens > 1 else dim
+    if copy is not None and (tuple(copy.shape) != (n_out, dim) or not copy.is_contiguous()):
+        raise KernelError(f"copy {tuple(copy.shape)} must be a contiguous [{n_out}, {dim}] tensor")
     lib = _build.load("groupnorm")
     _check(
         lib,
@@ -84,7 +87,8 @@ def group_rmsnorm(
             _ptr(gate), ctypes.c_int(_code(gate.dtype) if gate is not None else 0), ctypes.c_long(gate_ld),
             _ptr(weight), ctypes.c_int(_code(weight.dtype)), _ptr(out), ctypes.c_int(_code(out.dtype)),
             ctypes.c_long(out.stride(0) if n_out > 1 else dim), _ptr(rows), ctypes.c_int(n_out), ctypes.c_int(dim), ctypes.c_int(groups),
-            ctypes.c_float(eps), ctypes.c_int(int(accumulate)), _stream(),
+            ctypes.c_float(eps), ctypes.c_int(int(accumulate)), _ptr(copy), ctypes.c_int(_code(copy.dtype) if copy is not None else 0),
+            ctypes.c_long(dim), _stream(),
         ),
     )
     return out

@@ -67,9 +67,12 @@ class PostNormBlock(Block):
         else:
             mixer_cache = cache
             s = ops.cast_rows(h, act)
-        self.norm1.add_normed(h, self.mixer.forward(s, batch, mixer_cache, write_cache))
-        if self.feed_forward is not None:
-            self.norm2.add_normed(h, self.feed_forward.forward(ops.cast_rows(h, act), batch))
+        mixed = self.mixer.forward(s, batch, mixer_cache, write_cache)
+        if self.feed_forward is None:
+            self.norm1.add_normed(h, mixed)
+        else:
+            x = self.norm1.add_normed(h, mixed, also=act)  # the stream after the sum, as the feed-forward reads it
+            self.norm2.add_normed(h, self.feed_forward.forward(x, batch))
         return None
 
 

@@ -69,9 +69,15 @@ class GroupRMSNorm(Norm):
             ops.add_rows(h, delta)
         return ops.group_rmsnorm(h, self.weight, self.groups, self.eps, self.runtime.act_dtype, rows=rows)
 
-    def add_normed(self, h: torch.Tensor, y: torch.Tensor) -> None:
-        """h (float32 [T, D]) += norm(y) * weight; `y` is [T, D] or float32 partial sums [P, T, D]."""
-        ops.group_rmsnorm(y, self.weight, self.groups, self.eps, torch.float32, out=h, accumulate=True)
+    def add_normed(self, h: torch.Tensor, y: torch.Tensor, also: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+        """h (float32 [T, D]) += norm(y) * weight; `y` is [T, D] or float32 partial sums [P, T, D].  With `also` the
+        rows of h as they then stand are returned in that type as well (h itself if it is float32): what the next
+        sublayer reads, from the same kernel."""
+        copy = None
+        if also is not None and also != h.dtype:
+            copy = torch.empty(h.shape, dtype=also, device=h.device)
+        ops.group_rmsnorm(y, self.weight, self.groups, self.eps, torch.float32, out=h, accumulate=True, copy=copy)
+        return copy if copy is not None else (h if also is not None else None)
 
     def normalize_(self, x: torch.Tensor) -> torch.Tensor:
         """Rows of `x` ([T, D], the rows may lie apart) normalised in place."""

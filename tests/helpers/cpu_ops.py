@@ -174,7 +174,7 @@ def token_logprobs(logits, rows, targets):
 
 
 # ---- layers with group norms, token shift, a selective state space, a latent attention and routed experts ---- #
-def group_rmsnorm(x, weight, groups, eps, out_dtype, rows=None, out=None, accumulate=False, gate=None):
+def group_rmsnorm(x, weight, groups, eps, out_dtype, rows=None, out=None, accumulate=False, gate=None, copy=None):
     v = x.float().sum(0) if x.dim() == 3 else x.float()
     if gate is not None:
         g = gate.float()
@@ -190,6 +190,8 @@ def group_rmsnorm(x, weight, groups, eps, out_dtype, rows=None, out=None, accumu
         out += y.to(out.dtype)
     else:
         out.copy_(y.to(out.dtype))
+    if copy is not None:
+        copy.copy_(out.to(copy.dtype))
     return out
 
 

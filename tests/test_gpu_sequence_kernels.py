@@ -51,9 +51,11 @@ def test_group_norm_forms(dtype, dim, groups):
     parts = torch.randn(3, 7, dim)
     h = torch.randn(7, dim)
     hd = h.to(DEV)
-    ops.group_rmsnorm(parts.to(DEV), wd, groups, 1e-5, torch.float32, out=hd, accumulate=True)
+    also = torch.empty(7, dim, dtype=dtype, device=DEV)
+    ops.group_rmsnorm(parts.to(DEV), wd, groups, 1e-5, torch.float32, out=hd, accumulate=True, copy=also)
     want = cpu_ops.group_rmsnorm(parts, wr, groups, 1e-5, torch.float32, out=h.clone(), accumulate=True)
     _close(hd, want, torch.float32, "accumulate")
+    assert torch.equal(also, hd.to(dtype))  # the stream as it now stands, in the activation type
     # in place on columns of a wider tensor; the other columns stay
     wide = (torch.randn(7, dim + 40) * 2).to(DEV, dtype)
     keep = wide.clone()
