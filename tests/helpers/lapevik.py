@@ -50,7 +50,7 @@ TINY_Q = {
     "layers": [
         _attn(5, 12, 12, 28, 30, 20, 0.3, 500.0, 8, mlp=_moe(36, 3, 3)),
         _ssm(2, 40, 70, 2, 4, 2),
-        _attn(2, 32, 16, 16, 64, 48, 0.25, 250000.0, 16, mlp=_moe(16, 6, 2)),
+        _attn(2, 32, 16, 16, 64, 48, 0.25, 300000.0, 16, mlp=_moe(16, 6, 2)),
     ],
 }
 # a sharp softmax (large scale) over long sequences: one key far back, or just behind a page border, carries a token's
