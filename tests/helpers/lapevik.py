@@ -63,6 +63,16 @@ TINY_R = {
     ],
 }
 
+# wider, so that a prompt of some hundred tokens takes the kernels' shapes for many rows (library products, the
+# attention's long-portion kernel on a row of 128, segments of the recurrence, the grouped product through LDS)
+MEDIUM = {
+    "architecture": "Lapevik", "vocab": 300, "width": 256, "norm": {"eps": 1e-5, "groups": 4},
+    "layers": [
+        _ssm(8, 32, 64, 2, 2, 4, mlp=_moe(128, 2, 1)),
+        _attn(4, 32, 32, 64, 96, 64, 0.125, 10000.0, 32, mlp=_moe(64, 3, 2)),
+    ],
+}
+
 ALL = {"tiny_p": TINY_P, "tiny_q": TINY_Q, "tiny_r": TINY_R}
 
 

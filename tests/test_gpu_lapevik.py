@@ -119,6 +119,25 @@ def test_sharp_attention_and_slow_state_over_long_sequences(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_wider_layers_and_many_rows(tmp_path, dtype):
+    """Width 256 and prompts of 600 and 300 tokens: the kernels' shapes for many rows, whole, in large portions beside
+    each other, and with a tail of single tokens."""
+    config = lapevik.MEDIUM
+    folder = lapevik.make_folder(tmp_path, "medium", seed=9, config=config)
+    vocab = config["vocab"]
+    requests = {"a": traces.random_tokens(31, 600, vocab), "b": traces.random_tokens(32, 300, vocab)}
+    want = lapevik.expected(folder, requests, dtype)
+    side_by_side = [
+        {"step": 0, "entries": [{"id": "a", "tokens": requests["a"][:290], "want": list(range(290))}, {"id": "b", "tokens": requests["b"][:270], "want": list(range(270))}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": requests["a"][290:], "want": list(range(310))}, {"id": "b", "tokens": requests["b"][270:], "want": list(range(30))}], "end": ["a", "b"]},
+    ]
+    for steps in (traces.whole(requests), side_by_side, traces.tail_one_by_one(requests, tail=20)):
+        got, _, _ = run(folder, dtype, steps, requests, vocab, page_size=32)
+        for rid in requests:
+            lapevik.check(got[rid], want[rid], dtype, f"medium {dtype} {rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(folders, dtype):
     """Every token a step of its own from an empty cache and a zero state, for 300 steps."""
     name = "tiny_p"
