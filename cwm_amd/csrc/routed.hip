@@ -439,8 +439,8 @@ __global__ void __launch_bounds__(256) grouped_tiled_kernel(const bf16_t* __rest
     }
     src_w[i] = w + (size_t)expert * w_stride + (size_t)(col < N ? col : N - 1) * K + piece * 8;
   }
-  // two steps of operands on their way: what is fetched at the start of step k is put into LDS at the end of step k + 1
-  uint4 ra[2][4], rw[2][4];
+  // three steps of operands on their way: what is fetched at the start of step k is put into LDS at the end of step k + 2
+  uint4 ra[3][4], rw[3][4];
   auto fetch = [&](uint4 (&fa)[4], uint4 (&fw)[4], int k0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -501,20 +501,22 @@ __global__ void __launch_bounds__(256) grouped_tiled_kernel(const bf16_t* __rest
       }
     }
   };
+  const int steps = K / 64;
   fetch(ra[0], rw[0], 0);
   stage(ra[0], rw[0], 0);
-  fetch(ra[0], rw[0], 64);  // for step 1, staged at the end of step 0
+  fetch(ra[1], rw[1], 64);
+  fetch(ra[2], rw[2], 128);
   __syncthreads();
-  for (int k0 = 0; k0 < K; k0 += 128) {  // two steps a turn, so that the two register sets keep their names
-    fetch(ra[1], rw[1], k0 + 128);
-    multiply(0);
-    stage(ra[0], rw[0], 1);
-    __syncthreads();
-    if (k0 + 64 >= K) break;
-    fetch(ra[0], rw[0], k0 + 192);
-    multiply(1);
-    stage(ra[1], rw[1], 0);
-    __syncthreads();
+  for (int base = 0; base < steps; base += 6) {  // six steps a turn: register set step % 3 and buffer step % 2 keep their names
+#pragma unroll
+    for (int u = 0; u < 6; ++u) {
+      const int step = base + u;
+      if (step >= steps) break;
+      fetch(ra[u % 3], rw[u % 3], (step + 3) * 64);  // this set's step went into LDS a step ago
+      multiply(u % 2);
+      stage(ra[(u + 1) % 3], rw[(u + 1) % 3], (u + 1) % 2);
+      __syncthreads();
+    }
   }
 #pragma unroll
   for (int rt = 0; rt < 4; ++rt) {

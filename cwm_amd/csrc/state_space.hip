@@ -39,11 +39,13 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ in
                                                         const float* __restrict__ bias, float* state, long state_ld, long state_off,
                                                         const int* __restrict__ slots, const int* __restrict__ cu_q,
                                                         const int* __restrict__ seq_of_token, T* __restrict__ out, int channels,
-                                                        int taps, int n_slots) {
+                                                        int taps, int n_slots, int by_sequence) {
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= channels) return;
-  const int t = blockIdx.x;
-  const int b = seq_of_token[t];
+  // a block a token; or (by_sequence) a block a sequence, for its first tokens and its state alone, the other
+  // tokens being the other kernel's
+  const int b = by_sequence ? blockIdx.x : seq_of_token[blockIdx.x];
+  const int t = by_sequence ? cu_q[b] : blockIdx.x;
   const int first = cu_q[b];
   const int j = t - first;
   const int q = cu_q[b + 1] - first;
@@ -56,7 +58,7 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ in
     float acc = bc;
 #pragma unroll
     for (int k = 0; k < CONV_MAX_TAPS; ++k)
-      if (k < taps) acc += wk[k] * Elem<T>::load(in + (size_t)(t - (hist - k)) * in_ld + c);
+      if (k < taps) acc = fmaf(wk[k], Elem<T>::load(in + (size_t)(t - (hist - k)) * in_ld + c), acc);
     Elem<T>::store(out + (size_t)t * channels + c, silu_f32(acc));
     return;
   }
@@ -80,7 +82,7 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ in
     float acc = bc;
 #pragma unroll
     for (int k = 0; k < CONV_MAX_TAPS; ++k)
-      if (k < taps) acc += wk[k] * input(jj - (hist - k));
+      if (k < taps) acc = fmaf(wk[k], input(jj - (hist - k)), acc);
     Elem<T>::store(out + (size_t)(first + jj) * channels + c, silu_f32(acc));
   }
   if (st) {
@@ -93,21 +95,65 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ in
   }
 }
 
-extern "C" int cwm_conv_silu(const void* in, long in_ld, int dtype, const float* w, const float* bias, float* state, long state_ld,
+// The tokens that read no state (place >= taps - 1 in their portion), bfloat16, eight channels a thread: a tap's eight
+// inputs are one load of 16 bytes.  The sums run in the order of the kernel above.
+__global__ void __launch_bounds__(256) conv_silu_body_kernel(const bf16_t* __restrict__ in, long in_ld, const float* __restrict__ w_by_tap,
+                                                             const float* __restrict__ bias, const int* __restrict__ cu_q,
+                                                             const int* __restrict__ seq_of_token, bf16_t* __restrict__ out, int channels,
+                                                             int taps) {
+  const int c = 8 * (blockIdx.y * blockDim.x + threadIdx.x);
+  if (c >= channels) return;
+  const int t = blockIdx.x;
+  const int hist = taps - 1;
+  if (t - cu_q[seq_of_token[t]] < hist) return;
+  float acc[8];
+  {
+    const float4 b0 = *(const float4*)(bias + c), b1 = *(const float4*)(bias + c + 4);
+    acc[0] = b0.x, acc[1] = b0.y, acc[2] = b0.z, acc[3] = b0.w, acc[4] = b1.x, acc[5] = b1.y, acc[6] = b1.z, acc[7] = b1.w;
+  }
+#pragma unroll
+  for (int k = 0; k < CONV_MAX_TAPS; ++k) {
+    if (k < taps) {
+      Frag8 x;
+      x.u = *(const uint4*)(in + (size_t)(t - (hist - k)) * in_ld + c);
+      // the weights tap by tap ([taps][channels]): a thread's eight are 32 bytes, the threads' side by side
+      const float4 w0 = *(const float4*)(w_by_tap + (size_t)k * channels + c), w1 = *(const float4*)(w_by_tap + (size_t)k * channels + c + 4);
+      const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(wv[e], bf16_to_f32(x.h[e]), acc[e]);
+    }
+  }
+  uint4 o;
+  o.x = pack2_bf16(silu_f32(acc[0]), silu_f32(acc[1]));
+  o.y = pack2_bf16(silu_f32(acc[2]), silu_f32(acc[3]));
+  o.z = pack2_bf16(silu_f32(acc[4]), silu_f32(acc[5]));
+  o.w = pack2_bf16(silu_f32(acc[6]), silu_f32(acc[7]));
+  *(uint4*)(out + (size_t)t * channels + c) = o;
+}
+
+// w_by_tap: the same weights as [taps][channels], or null (then every token goes through the kernel of a thread a channel)
+extern "C" int cwm_conv_silu(const void* in, long in_ld, int dtype, const float* w, const float* w_by_tap, const float* bias, float* state, long state_ld,
                              long state_off, const int* slots, const int* cu_q, const int* seq_of_token, void* out, int n_tokens,
-                             int channels, int taps, int n_slots, hipStream_t stream) {
+                             int n_seqs, int channels, int taps, int n_slots, hipStream_t stream) {
   CWM_REQUIRE(in && w && bias && state && slots && cu_q && seq_of_token && out, "conv_silu: arguments missing");
   CWM_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "conv_silu: %d taps, the kernel takes 1..%d", taps, CONV_MAX_TAPS);
   CWM_REQUIRE(channels > 0 && in_ld >= channels && n_tokens >= 0, "conv_silu: bad sizes");
   CWM_REQUIRE(state_off >= 0 && state_off + (long)(taps - 1) * channels <= state_ld, "conv_silu: the state row is too short");
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, (channels + 255) / 256);
-  if (dtype == CWM_BF16)
+  if (dtype == CWM_BF16 && w_by_tap && n_seqs > 0 && n_tokens > n_seqs && channels % 8 == 0 && in_ld % 8 == 0 && ((uintptr_t)in % 16) == 0 &&
+      ((uintptr_t)out % 16) == 0 && ((uintptr_t)w_by_tap % 16) == 0 && ((uintptr_t)bias % 16) == 0) {
+    // portions of a prompt: the tokens that read no state in pieces of 16 bytes, then a block a sequence for the rest
+    hipLaunchKernelGGL(conv_silu_body_kernel, dim3(n_tokens, (channels / 8 + 255) / 256), dim3(256), 0, stream, (const bf16_t*)in, in_ld, w_by_tap,
+                       bias, cu_q, seq_of_token, (bf16_t*)out, channels, taps);
+    hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, dim3(n_seqs, (channels + 255) / 256), dim3(256), 0, stream, (const bf16_t*)in, in_ld, w, bias,
+                       state, state_ld, state_off, slots, cu_q, seq_of_token, (bf16_t*)out, channels, taps, n_slots, 1);
+  } else if (dtype == CWM_BF16)
     hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)in, in_ld, w, bias, state, state_ld, state_off,
-                       slots, cu_q, seq_of_token, (bf16_t*)out, channels, taps, n_slots);
+                       slots, cu_q, seq_of_token, (bf16_t*)out, channels, taps, n_slots, 0);
   else if (dtype == CWM_F32)
     hipLaunchKernelGGL(conv_silu_kernel<float>, grid, dim3(256), 0, stream, (const float*)in, in_ld, w, bias, state, state_ld, state_off,
-                       slots, cu_q, seq_of_token, (float*)out, channels, taps, n_slots);
+                       slots, cu_q, seq_of_token, (float*)out, channels, taps, n_slots, 0);
   else
     return cwm_fail("conv_silu: unknown dtype %d", dtype);
   return cwm_launch_status("conv_silu");

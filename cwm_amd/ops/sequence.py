@@ -161,7 +161,10 @@ def sigmoid_mul(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, state_offset: int, batch: Any) -> torch.Tensor:
+def causal_conv_silu(
+    x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, state_offset: int, batch: Any,
+    weight_by_tap: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
     """silu(bias + causal convolution) per channel over each sequence of the step: `x` [T, C] (rows may lie apart),
     `weight` float32 [C, taps] (the last column is the current token's), `bias` float32 [C].  A sequence's last
     taps - 1 inputs live in its row of `state` (float32 [slots, n]) from `state_offset` on, [taps - 1, C] oldest
@@ -186,9 +189,9 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, 
     _check(
         lib,
         lib.cwm_conv_silu(
-            _ptr(x), ctypes.c_long(x.stride(0) if n_tokens > 1 else channels), ctypes.c_int(_code(x.dtype)), _ptr(weight), _ptr(bias),
+            _ptr(x), ctypes.c_long(x.stride(0) if n_tokens > 1 else channels), ctypes.c_int(_code(x.dtype)), _ptr(weight), _ptr(weight_by_tap), _ptr(bias),
             _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_long(state_offset), _ptr(batch.state_slots), _ptr(batch.cu_q),
-            _ptr(batch.seq_of_token), _ptr(out), ctypes.c_int(n_tokens), ctypes.c_int(channels), ctypes.c_int(taps),
+            _ptr(batch.seq_of_token), _ptr(out), ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs), ctypes.c_int(channels), ctypes.c_int(taps),
             ctypes.c_int(state.shape[0]), _stream(),
         ),
     )

@@ -61,6 +61,7 @@ class SelectiveStateSpace(Mixer):
         self.w_out = LinearWeights(tensors["o"], stream_copy=runtime.stream_copies)
         # everything that enters the recurrence is kept in float32 (exact from a 16-bit file)
         self.conv_w = tensors["conv"].float().contiguous()
+        self.conv_w_by_tap = self.conv_w.t().contiguous()  # [taps, channels]: what portions of a prompt read
         self.conv_b = tensors["conv.b"].float().contiguous()
         self.dt_bias = tensors["dt_bias"].float().contiguous()
         self.a_log = tensors["A_log"].float().contiguous()
@@ -73,7 +74,7 @@ class SelectiveStateSpace(Mixer):
         inner = self.inner
         z = u[:, :inner]
         xbc = ops.causal_conv_silu(
-            u[:, inner : inner + self.channels], self.conv_w, self.conv_b, cache.state, self.ssm_elems, batch,
+            u[:, inner : inner + self.channels], self.conv_w, self.conv_b, cache.state, self.ssm_elems, batch, self.conv_w_by_tap,
         )
         y = ops.selective_scan(
             xbc, u[:, inner + self.channels :], self.dt_bias, self.a_log, self.d_skip, cache.state, batch,

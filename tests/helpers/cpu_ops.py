@@ -216,7 +216,7 @@ def sigmoid_mul(a, gate):
     return (a.float() * torch.sigmoid(gate.float())).to(a.dtype)
 
 
-def causal_conv_silu(x, weight, bias, state, state_offset, batch):
+def causal_conv_silu(x, weight, bias, state, state_offset, batch, weight_by_tap=None):
     taps, channels = weight.shape[1], x.shape[1]
     out = torch.empty(x.shape, dtype=torch.float32)
     for b in range(batch.n_seqs):

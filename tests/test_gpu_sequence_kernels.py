@@ -90,12 +90,14 @@ def test_token_shift_first_tokens_and_state(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
-def test_causal_conv_against_whole_sequence(dtype, taps):
-    """Portions of 1, 2, 3 and more tokens carry the convolution's inputs through the state."""
+@pytest.mark.parametrize("channels", [300, 320])
+def test_causal_conv_against_whole_sequence(dtype, taps, channels):
+    """Portions of 1, 2, 3 and more tokens carry the convolution's inputs through the state (320 channels in rows of a
+    multiple of 16 bytes: the path that fetches eight channels at once)."""
     from cwm_amd import ops
 
     torch.manual_seed(taps)
-    channels, offset, n = 300, 17, 23
+    offset, n = 17, 23
     x = torch.randn(n, channels).to(dtype)
     w, b = torch.randn(channels, taps), torch.randn(channels)
     whole_state = torch.zeros(2, offset + (taps - 1) * channels + 5)
@@ -104,9 +106,10 @@ def test_causal_conv_against_whole_sequence(dtype, taps):
     state[0] = 7.0  # another request's slot
     at, outs = 0, []
     for q in (1, 2, 1, 3, 9, 2, 5):
-        wide = torch.randn(q, channels + 10).to(DEV, dtype)  # rows that lie apart
-        wide[:, 3 : 3 + channels] = x[at : at + q].to(DEV)
-        outs.append(ops.causal_conv_silu(wide[:, 3 : 3 + channels], w.to(DEV), b.to(DEV), state, offset, _batch([q], [at], [1], DEV)))
+        lead = 3 if channels % 8 else 8
+        wide = torch.randn(q, channels + 16).to(DEV, dtype)  # rows that lie apart
+        wide[:, lead : lead + channels] = x[at : at + q].to(DEV)
+        outs.append(ops.causal_conv_silu(wide[:, lead : lead + channels], w.to(DEV), b.to(DEV), state, offset, _batch([q], [at], [1], DEV), w.t().contiguous().to(DEV)))
         at += q
     _close(torch.cat(outs), whole, dtype, "portions")
     _close(state[1], whole_state[1], torch.float32, "state")
