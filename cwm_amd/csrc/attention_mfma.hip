@@ -149,7 +149,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
                       const bf16_t* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                       const int* __restrict__ cu_q, const int* __restrict__ kv_len, const int* __restrict__ work,
                       int n_work, float* __restrict__ partial, int n_q_heads, int n_kv_heads, int page_size,
-                      int page_shift, int num_pages, int window_left, float scale_log2e) {
+                      int page_shift, int num_pages, int window_left, float scale_log2e, const float* __restrict__ sink) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int id = blockIdx.x;  // (item, key/value head): the same for the whole block
@@ -370,6 +370,9 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   for (int dt = 0; dt < D_TILES; ++dt) *(float4v*)&team_o[wave][n][16 * dt + 4 * j] = acc[dt] * mine;
   __syncthreads();
   if (!row_valid) return;
+  // a sink: one more term of the denominator, exp(sink) of the query head (not scaled, no key, no value).  It
+  // counts once a row: a block that leaves a partial result leaves it to the merge kernel
+  if (sink && slot < 0) l_all += __builtin_amdgcn_exp2f(sink[hq] * 1.4426950408889634f - m_all * scale_log2e);
   const float inv = page_missing ? not_a_number() : 1.0f / l_all;
   bf16_t* orow = out + (size_t)(q0 + ti) * out_stride + (size_t)hq * HEAD_DIM;
   float* prow = slot < 0 ? nullptr : partial + (((size_t)slot * n_kv_heads + g) * 16 + n) * PARTIAL_STRIDE;
@@ -450,7 +453,7 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
                      const bf16_t* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                      const int* __restrict__ cu_q, const int* __restrict__ kv_len, const int* __restrict__ work,
                      float* __restrict__ partial, int n_kv_heads_grid, int n_q_heads, int n_kv_heads, int page_size,
-                     int page_shift, int num_pages, int window_left, float scale_log2e) {
+                     int page_shift, int num_pages, int window_left, float scale_log2e, const float* __restrict__ sink) {
   constexpr bool FAST = MODE != LDS_PLAIN;
   constexpr int DMA_AHEAD = DMA_BUFFERS - 1;
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[MODE == LDS_DMA ? 1 : 2][MODE == LDS_DMA ? 8 : 32 * LDS_K_STRIDE];
@@ -878,6 +881,7 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
       }
       continue;
     }
+    if (sink) l_row += __builtin_amdgcn_exp2f(sink[hq[rt]] * 1.4426950408889634f - m_run[rt] * scale_log2e);
     const float inv = page_missing ? not_a_number() : 1.0f / l_row;
     bf16_t* orow = out + (size_t)(q0 + ti[rt]) * out_stride + (size_t)hq[rt] * HEAD_DIM;
 #pragma unroll
@@ -899,7 +903,8 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
 template <int MERGE_WAVES>
 __global__ void __launch_bounds__(MERGE_WAVES * 64)
 attention_merge_kernel(bf16_t* __restrict__ out, long out_stride, const float* __restrict__ partial,
-                       const int* __restrict__ cu_q, const int* __restrict__ merge, int n_q_heads, int n_kv_heads) {
+                       const int* __restrict__ cu_q, const int* __restrict__ merge, int n_q_heads, int n_kv_heads,
+                       const float* __restrict__ sink) {
   __shared__ float red_max[MERGE_WAVES];
   __shared__ float red_l[MERGE_WAVES];
   __shared__ float red_o[MERGE_WAVES][HEAD_DIM];
@@ -960,6 +965,7 @@ attention_merge_kernel(bf16_t* __restrict__ out, long out_stride, const float* _
   float l_all = 0.f;
 #pragma unroll
   for (int w = 0; w < MERGE_WAVES; ++w) l_all += red_l[w];
+  if (sink) l_all += exp2f(sink[hq] * 1.4426950408889634f - m_all);  // the maxima are kept in the scaled (log2) domain
   const float inv = 1.0f / l_all;
   bf16_t* orow = out + (size_t)(q0 + ti) * out_stride + (size_t)hq * HEAD_DIM;
 #pragma unroll
@@ -979,7 +985,8 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
                                   const int* work, int n_work, int work_keys, const int* work_wide, int n_work_wide, int wide_tiles,
                                   int wide_three_blocks, const int* merge,
                                   int n_merge, int n_merge_mid, int n_merge_few, float* partial, int n_q_heads, int n_kv_heads, int head_dim,
-                                  int page_size, int num_pages, int window_left, float scale, hipStream_t stream) {
+                                  int page_size, int num_pages, int window_left, float scale, const float* sink,
+                                  hipStream_t stream) {
   // `work`: items of one 16-row tile (may be split over chunks of keys), one wavefront each;
   // `work_wide`: items of 4 * LDS_RT row tiles, one block each with keys and values in LDS
   CWM_REQUIRE(head_dim == HEAD_DIM, "attention_mfma: this library is built for head_dim %d, not %d", HEAD_DIM, head_dim);
@@ -1008,7 +1015,7 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
   hipLaunchKernelGGL((attention_mfma_kernel<PAGE32>), dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16_t*)q,     \
                      q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, cu_q, kv_len,   \
                      work, n_work, partial, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left,        \
-                     scale_log2e)
+                     scale_log2e, sink)
     if (page_size % 32 == 0)
       CWM_LAUNCH_TEAM(true);
     else
@@ -1024,7 +1031,7 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
   hipLaunchKernelGGL((attention_lds_kernel<MODE, BUFFERS, MIN_BLOCKS>), dim3((unsigned)blocks), dim3(256), 0, stream,     \
                      (const bf16_t*)q, q_stride,                                                                          \
                      (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, cu_q, kv_len, work_wide,   \
-                     partial, n_kv_heads, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left, scale_log2e)
+                     partial, n_kv_heads, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left, scale_log2e, sink)
     // tiles of 32 keys that never straddle a page, and shares of a tile that divide evenly over the block
     if (page_size % 32 == 0 && LDS_K_CHUNKS % 256 == 0 && LDS_V_CHUNKS % 256 == 0) {
 #if DMA_HEAD_DIM_OK
@@ -1054,7 +1061,7 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
 #define CWM_LAUNCH_MERGE(WAVES, COUNT, FIRST)                                                                              \
   if ((COUNT) > 0)                                                                                                        \
   hipLaunchKernelGGL(attention_merge_kernel<WAVES>, dim3(COUNT, n_kv_heads, 16), dim3(WAVES * 64), 0, stream, (bf16_t*)out, \
-                     out_stride, (const float*)partial, cu_q, merge + (size_t)(FIRST) * 4, n_q_heads, n_kv_heads)
+                     out_stride, (const float*)partial, cu_q, merge + (size_t)(FIRST) * 4, n_q_heads, n_kv_heads, sink)
     CWM_LAUNCH_MERGE(16, n_many, 0);
     CWM_LAUNCH_MERGE(4, n_merge_mid, n_many);
     CWM_LAUNCH_MERGE(1, n_merge_few, n_many + n_merge_mid);

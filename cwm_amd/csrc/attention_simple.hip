@@ -67,7 +67,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
                         const T* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token, float* __restrict__ partial,
                         int n_q_heads, int n_kv_heads, int head_groups, int head_dim, int page_size, int num_pages,
-                        int window_left, float scale) {
+                        int window_left, float scale, const float* __restrict__ sink) {
   __shared__ __attribute__((aligned(16))) float qs[HEADS][D_REGS * CWM_WAVE];
   // probabilities of a chunk, key jj at [in0 + jj] (in0: the first key's place in its block of 8 values), so that the
   // eight of a block lie at a multiple of 8
@@ -316,6 +316,9 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
       weight[w] = (part_m[w][h] == neg_inf) ? 0.f : expf(part_m[w][h] - m_all);  // -inf: that wavefront had no chunk
       l_all += part_l[w][h] * weight[w];
     }
+    // a sink is one more term of the denominator, exp(sink) of the query head, with no key and no value; it
+    // counts once for the token, so where the token has several segments the join kernel adds it
+    if (sink && n_seg == 1) l_all += expf(sink[h0 + h] - m_all);
     T* orow = out + (size_t)t * out_stride + (size_t)(h0 + h) * head_dim;
     float* prow = n_seg > 1 ? partial + (((size_t)t * n_q_heads + h0 + h) * SIMPLE_MAX_SEGMENTS + seg) * PARTIAL_STRIDE(head_dim) : nullptr;
 #pragma unroll
@@ -344,7 +347,7 @@ template <typename T>
 __global__ void __launch_bounds__(CWM_WAVE)
 attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ partial,
                              const int* __restrict__ positions, int n_q_heads, int head_dim, int window_left,
-                             int max_segments) {
+                             int max_segments, const float* __restrict__ sink) {
   const int t = blockIdx.x / n_q_heads;
   const int h = blockIdx.x - t * n_q_heads;
   const int lane = threadIdx.x;
@@ -372,6 +375,7 @@ attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* 
       if (d < head_dim) o[r] += prow[d] * weight;
     }
   }
+  if (sink) l_all += expf(sink[h] - m_all);
   T* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
 #pragma unroll
   for (int r = 0; r < SIMPLE_D_REGS; ++r) {
@@ -381,14 +385,15 @@ attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* 
 }
 
 // `max_keys`: the most keys that any token of the call reads (its position + 1, or the window if that
-// is less); `partial`: float32 scratch of n_tokens * n_q_heads * 16 * (head_dim + 2) values, needed
+// is less); `sink`: null, or float32 [n_q_heads], a term exp(sink) of every softmax denominator that has no key and
+// no value (it is not scaled and counts once a token); `partial`: float32 scratch of n_tokens * n_q_heads * 16 * (head_dim + 2) values, needed
 // (and touched) only if max_keys exceeds 2,048.  A token that reads more keys than `max_keys` says has no
 // place for its segments' results: its rows of `out` are NaN and every kernel ends normally.
 extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, long out_stride, const void* cache,
                                     int dtype, const int* block_table, int table_width, const int* positions,
                                     const int* seq_of_token, int n_tokens, int n_q_heads, int n_kv_heads,
                                     int head_dim, int page_size, int num_pages, int window_left, float scale,
-                                    int max_keys, float* partial, hipStream_t stream) {
+                                    int max_keys, float* partial, const float* sink, hipStream_t stream) {
   CWM_REQUIRE(n_tokens >= 0, "attention: negative token count");
   CWM_REQUIRE(head_dim > 0 && head_dim <= SIMPLE_MAX_HEAD_DIM, "attention: head_dim %d is outside 1..%d", head_dim,
               SIMPLE_MAX_HEAD_DIM);
@@ -416,7 +421,7 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
   hipLaunchKernelGGL((attention_simple_kernel<float, HEADS, D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream,     \
                      (const float*)q, q_stride, (float*)out, out_stride, (const float*)cache, block_table, table_width,   \
                      positions, seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, \
-                     window_left, scale)
+                     window_left, scale, sink)
 #define CWM_LAUNCH_SIMPLE_HEADS(D_REGS)   \
   do {                                    \
     if (heads <= 2)                       \
@@ -438,15 +443,15 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
 #undef CWM_LAUNCH_SIMPLE
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<float>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
-                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments);
+                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments, sink);
   } else if (dtype == CWM_BF16) {
     hipLaunchKernelGGL((attention_simple_kernel<bf16_t, SIMPLE_HEADS, SIMPLE_D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const bf16_t*)q,
                        q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, positions,
                        seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, window_left,
-                       scale);
+                       scale, sink);
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<bf16_t>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
-                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments);
+                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments, sink);
   } else {
     return cwm_fail("attention: unknown dtype %d", dtype);
   }

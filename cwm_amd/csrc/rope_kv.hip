@@ -275,3 +275,144 @@ extern "C" int cwm_rope_kv_write_partials(void* qkv, long qkv_stride, const floa
                      num_pages, n_q_heads, n_kv_heads, head_dim, partials, n_partials, partial_stride);
   return cwm_launch_status("rope_kv_write_partials");
 }
+
+// ---- projection rows -> norm over the whole projection -> rotation -> cache ---------------------------- //
+// A token's row of the joined projection is [q: Hq * qk_dim | k: Hkv * qk_dim | v: Hkv * v_dim] (type TS, or float32
+// partial sums of a split K, added in order).  Queries and keys are each divided by the root mean square of the
+// whole projection (all heads at once, eps inside the root) and multiplied by a weight per element, where a weight
+// is given; then their heads are rotated by position * inv_freq[pair] (adjacent pairs; a frequency of 0 leaves its
+// pair alone, so a table that ends in zeros rotates the leading dimensions only).  Heads are then laid out with
+// `head_dim` elements, the common size of a cached key and value: a key's elements from qk_dim on and a value's
+// from v_dim on are zeros (a zero adds nothing to a score, and the output columns it makes are dropped by the
+// caller).  Queries go to q_out [T][Hq][head_dim], keys and values into the paged cache (layout at the top of
+// this file).  All arithmetic float32; one block a token.
+#define NORM_ROPE_MAX_HEAD 256
+template <typename TS, typename TO>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_write_kernel(const TS* __restrict__ src, long src_stride, int n_partials, long partial_stride,
+                          TO* __restrict__ q_out, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+                          float eps, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                          const float* __restrict__ inv_freq, TO* __restrict__ cache, const int* __restrict__ block_table,
+                          int table_width, int page_size, int num_pages, int n_q_heads, int n_kv_heads, int qk_dim,
+                          int v_dim, int head_dim) {
+  __shared__ float scratch[16];
+  __shared__ float cs[NORM_ROPE_MAX_HEAD];  // cos, sin of each pair
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = head_dim / 2;
+  const int q_width = n_q_heads * qk_dim, k_width = n_kv_heads * qk_dim;
+  const TS* srow = src + (size_t)t * src_stride;
+  auto value = [&](int e) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += Elem<TS>::load(srow + (size_t)p * partial_stride + e);
+    return v;
+  };
+  TO* kdst = nullptr;
+  TO* vdst = nullptr;
+  int slot = 0;
+  if (cache) {
+    const int seq = seq_of_token[t];
+    const int lp = pos / page_size;
+    slot = pos - lp * page_size;
+    const int page = (lp >= 0 && lp < table_width) ? block_table[(size_t)seq * table_width + lp] : -1;
+    if (page >= 0 && page < num_pages) {
+      const size_t plane = (size_t)n_kv_heads * page_size * head_dim;
+      kdst = cache + (size_t)page * 2 * plane;
+      vdst = kdst + plane;
+    }
+  }
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float c = 1.f, s = 0.f;
+    const float f = inv_freq ? inv_freq[i] : 0.f;
+    if (f != 0.f) sincosf((float)pos * f, &s, &c);
+    cs[2 * i] = c;
+    cs[2 * i + 1] = s;
+  }
+  float q_rstd = 1.f, k_rstd = 1.f;
+  if (q_weight) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < q_width; e += blockDim.x) {
+      const float v = value(e);
+      ss += v * v;
+    }
+    q_rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)q_width + eps);
+  }
+  if (k_weight && cache) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < k_width; e += blockDim.x) {
+      const float v = value(q_width + e);
+      ss += v * v;
+    }
+    k_rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)k_width + eps);
+  }
+  __syncthreads();  // the table of cosines and sines is complete
+  const int n_heads = n_q_heads + (cache ? n_kv_heads : 0);
+  for (int e = threadIdx.x; e < n_heads * half; e += blockDim.x) {
+    const int hh = e / half, i = e - hh * half;
+    const bool is_key = hh >= n_q_heads;
+    const int head = is_key ? hh - n_q_heads : hh;
+    const int base = (is_key ? q_width : 0) + head * qk_dim;
+    const float* weight = is_key ? k_weight : q_weight;
+    const float rstd = is_key ? k_rstd : q_rstd;
+    float re = 0.f, im = 0.f;
+    if (2 * i < qk_dim) re = value(base + 2 * i) * (weight ? rstd * weight[head * qk_dim + 2 * i] : 1.f);
+    if (2 * i + 1 < qk_dim) im = value(base + 2 * i + 1) * (weight ? rstd * weight[head * qk_dim + 2 * i + 1] : 1.f);
+    const float c = cs[2 * i], s = cs[2 * i + 1];
+    const float ore = re * c - im * s, oim = im * c + re * s;
+    TO* dst = nullptr;
+    if (!is_key)
+      dst = q_out + ((size_t)t * n_q_heads + head) * head_dim;
+    else if (kdst)
+      dst = kdst + ((size_t)head * page_size + slot) * head_dim;
+    if (dst) {
+      Elem<TO>::store(dst + 2 * i, ore);
+      Elem<TO>::store(dst + 2 * i + 1, oim);
+    }
+  }
+  if (vdst) {
+    const int v_block = (page_size % 8 == 0) ? 8 : page_size;
+    const int v_base = q_width + k_width;
+    for (int e = threadIdx.x; e < n_kv_heads * head_dim; e += blockDim.x) {
+      const int head = e / head_dim, d = e - head * head_dim;
+      const float v = d < v_dim ? value(v_base + head * v_dim + d) : 0.f;
+      Elem<TO>::store(vdst + (size_t)head * head_dim * page_size + ((size_t)(slot / v_block) * head_dim + d) * v_block + slot % v_block, v);
+    }
+  }
+}
+
+// src: [n_tokens][src_stride] of src_dtype, or n_partials float32 slabs partial_stride apart.  q_weight [Hq * qk_dim],
+// k_weight [Hkv * qk_dim]: float32, null for no norm.  inv_freq: float32 [head_dim / 2] or null.  cache: null where
+// only the queries are wanted (a layer that reads a cache written by another).
+extern "C" int cwm_qk_norm_rope_write(const void* src, int src_dtype, long src_stride, int n_partials, long partial_stride,
+                                      void* q_out, int out_dtype, const float* q_weight, const float* k_weight, float eps,
+                                      const int* positions, const int* seq_of_token, const float* inv_freq, void* cache,
+                                      const int* block_table, int table_width, int page_size, int num_pages, int n_tokens,
+                                      int n_q_heads, int n_kv_heads, int qk_dim, int v_dim, int head_dim, hipStream_t stream) {
+  CWM_REQUIRE(n_tokens >= 0 && n_partials >= 1, "qk_norm_rope_write: bad sizes");
+  CWM_REQUIRE(n_partials == 1 || src_dtype == CWM_F32, "qk_norm_rope_write: partial sums must be float32");
+  CWM_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= NORM_ROPE_MAX_HEAD,
+              "qk_norm_rope_write: head_dim %d must be even and at most %d", head_dim, NORM_ROPE_MAX_HEAD);
+  CWM_REQUIRE(qk_dim >= 1 && v_dim >= 1 && qk_dim <= head_dim && v_dim <= head_dim,
+              "qk_norm_rope_write: heads of %d (queries, keys) and %d (values) do not fit the cached head of %d", qk_dim, v_dim, head_dim);
+  CWM_REQUIRE(n_q_heads > 0 && n_kv_heads > 0, "qk_norm_rope_write: no heads");
+  CWM_REQUIRE(src && q_out && positions, "qk_norm_rope_write: arguments missing");
+  CWM_REQUIRE(eps > 0.f || (!q_weight && !k_weight), "qk_norm_rope_write: eps must be positive");
+  if (cache) {
+    CWM_REQUIRE(block_table && seq_of_token, "qk_norm_rope_write: a cache write needs a block table");
+    CWM_REQUIRE(page_size > 0 && num_pages > 0 && table_width > 0, "qk_norm_rope_write: bad cache geometry");
+  }
+  if (n_tokens == 0) return 0;
+  const int key = (src_dtype << 1) | out_dtype;
+#define CWM_NORM_ROPE(TS, TO)                                                                                               \
+  hipLaunchKernelGGL((qk_norm_rope_write_kernel<TS, TO>), dim3(n_tokens), dim3(256), 0, stream, (const TS*)src, src_stride, \
+                     n_partials, partial_stride, (TO*)q_out, q_weight, k_weight, eps, positions, seq_of_token, inv_freq,    \
+                     (TO*)cache, block_table, table_width, page_size, num_pages, n_q_heads, n_kv_heads, qk_dim, v_dim, head_dim)
+  switch (key) {
+    case 0: CWM_NORM_ROPE(float, float); break;
+    case 1: CWM_NORM_ROPE(float, bf16_t); break;
+    case 3: CWM_NORM_ROPE(bf16_t, bf16_t); break;
+    default: return cwm_fail("qk_norm_rope_write: source type %d with cache type %d is not built", src_dtype, out_dtype);
+  }
+#undef CWM_NORM_ROPE
+  return cwm_launch_status("qk_norm_rope_write");
+}

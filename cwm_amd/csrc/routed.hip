@@ -1,7 +1,8 @@
 // Routed experts and other products in which every row has a weight matrix of its own choosing.
 //
 //   route_top        per token: the `top` largest of its router logits (the lower index wins a tie) and the softmax
-//                    over those alone, float32.
+//                    over those alone, float32; or, mode 1, the softmax over all experts, a choice by score plus a
+//                    correction per expert, and weights that are the chosen scores times a scale.
 //   group_by_expert  the step's (token, choice) pairs grouped by expert, each group padded to whole tiles of 16
 //                    rows: row_token[row] (-1 in the padding), pair_row[pair], tile_expert[tile] (-1 beyond the
 //                    last tile).  One block; no count leaves the device.  The order of a group's rows is whatever
@@ -10,7 +11,7 @@
 //                    or, for a batch of independent products (one weight per head, say), from the block's z.
 //                    bfloat16 operands on v_mfma_f32_16x16x32_bf16, float32 operands on v_mfma_f32_16x16x4_f32
 //                    (exact products); float32 sums in the order of k either way, whatever else is in the step.
-//                    With two weights the epilogue forms silu(W0 a) * (W1 a).
+//                    With two weights the epilogue forms silu(W0 a) * (W1 a), or the clamped form of `GateAct`.
 //   combine          out[t] = sum_k weight[t][k] * rows[pair_row[t][k]] in the order of k, float32.
 //
 // Matrix-core layout as in the other products of this package: operand A = the weight tile (lane 16 j + r: row
@@ -28,11 +29,23 @@ extern "C" int cwm_route_max_top() { return ROUTE_MAX_TOP; }
 extern "C" int cwm_route_max_experts() { return ROUTE_MAX_EXPERTS; }
 extern "C" int cwm_route_tile_rows() { return TILE_ROWS; }
 
+// mode 0: the `top` largest logits, weights = softmax over those alone.
+// mode 1: scores s = softmax over all experts; the `top` largest of s + correction (correction: null for none) are
+//         chosen; weights = scale * s of the chosen, divided by their sum first if `renormalize`.
 __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ chosen,
-                                                        float* __restrict__ weights, int n_tokens, int n_experts, int top) {
+                                                        float* __restrict__ weights, int n_tokens, int n_experts, int top, int mode,
+                                                        const float* __restrict__ correction, float scale, int renormalize) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n_tokens) return;
   const float* z = logits + (size_t)t * n_experts;
+  float largest_all = 0.f, inv_all = 1.f;
+  if (mode == 1) {
+    largest_all = z[0];
+    for (int e = 1; e < n_experts; ++e) largest_all = fmaxf(largest_all, z[e]);
+    float sum_all = 0.f;
+    for (int e = 0; e < n_experts; ++e) sum_all += expf(z[e] - largest_all);
+    inv_all = 1.f / sum_all;
+  }
   int idx[ROUTE_MAX_TOP];
   float val[ROUTE_MAX_TOP];
 #pragma unroll
@@ -44,44 +57,58 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
   for (int k = 0; k < ROUTE_MAX_TOP; ++k) {
     if (k < top) {
       int best = -1;
-      float bv = 0.f;
+      float bv = 0.f, bs = 0.f;
       for (int e = 0; e < n_experts; ++e) {
         bool taken = false;
 #pragma unroll
         for (int m = 0; m < ROUTE_MAX_TOP; ++m) taken |= (m < k && idx[m] == e);
-        const float v = z[e];
+        float v = z[e], score = v;
+        if (mode == 1) {
+          score = expf(v - largest_all) * inv_all;
+          v = correction ? score + correction[e] : score;
+        }
         if (!taken && (best < 0 || v > bv)) {
           best = e;
           bv = v;
+          bs = score;
         }
       }
       idx[k] = best;
-      val[k] = bv;
+      val[k] = mode == 1 ? bs : bv;
     }
   }
   float sum = 0.f;
-  const float largest = val[0];  // the first chosen is the largest
+  if (mode == 0) {
+    const float largest = val[0];  // the first chosen is the largest
 #pragma unroll
-  for (int k = 0; k < ROUTE_MAX_TOP; ++k)
-    if (k < top) {
-      val[k] = expf(val[k] - largest);
-      sum += val[k];
-    }
+    for (int k = 0; k < ROUTE_MAX_TOP; ++k)
+      if (k < top) {
+        val[k] = expf(val[k] - largest);
+        sum += val[k];
+      }
+  } else {
+#pragma unroll
+    for (int k = 0; k < ROUTE_MAX_TOP; ++k)
+      if (k < top) sum += val[k];
+    if (!renormalize) sum = 1.f;
+  }
 #pragma unroll
   for (int k = 0; k < ROUTE_MAX_TOP; ++k)
     if (k < top) {
       chosen[(size_t)t * top + k] = idx[k];
-      weights[(size_t)t * top + k] = val[k] / sum;
+      weights[(size_t)t * top + k] = mode == 0 ? val[k] / sum : scale * (val[k] / sum);
     }
 }
 
-extern "C" int cwm_route_top(const float* logits, int* chosen, float* weights, int n_tokens, int n_experts, int top,
-                             hipStream_t stream) {
+extern "C" int cwm_route_top(const float* logits, int* chosen, float* weights, int n_tokens, int n_experts, int top, int mode,
+                             const float* correction, float scale, int renormalize, hipStream_t stream) {
   CWM_REQUIRE(logits && chosen && weights, "route_top: arguments missing");
   CWM_REQUIRE(top >= 1 && top <= ROUTE_MAX_TOP && top <= n_experts, "route_top: %d of %d experts, the kernel takes up to %d", top, n_experts,
               ROUTE_MAX_TOP);
+  CWM_REQUIRE(mode == 0 || mode == 1, "route_top: unknown mode %d", mode);
   if (n_tokens <= 0) return 0;
-  hipLaunchKernelGGL(route_top_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, stream, logits, chosen, weights, n_tokens, n_experts, top);
+  hipLaunchKernelGGL(route_top_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, stream, logits, chosen, weights, n_tokens, n_experts, top,
+                     mode, correction, scale, renormalize);
   return cwm_launch_status("route_top");
 }
 
@@ -140,6 +167,22 @@ extern "C" int cwm_group_by_expert(const int* chosen, int n_tokens, int top, int
 }
 
 // ---- the grouped product ------------------------------------------------------------------------------------- //
+// What the epilogue of a product with two weights makes of g = W0 a and u = W1 a:
+//   kind 0: silu(g) * u
+//   kind 1: g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
+struct GateAct {
+  int kind;
+  float alpha, limit;
+};
+__device__ __forceinline__ float gated_value(float g, float u, const GateAct act) {
+  if (act.kind == 1) {
+    g = fminf(g, act.limit);
+    u = fminf(fmaxf(u, -act.limit), act.limit);
+    return g / (1.f + expf(-act.alpha * g)) * (u + 1.f);
+  }
+  return g / (1.f + expf(-g)) * u;
+}
+
 template <typename T> struct Frag;
 template <> struct Frag<bf16_t> {
   static constexpr int K_STEP = 32;  // values of k one matrix instruction takes
@@ -188,7 +231,7 @@ template <typename T, int RT, int CT, int WR, bool GATED, bool VEC>
 __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
                                                               const T* __restrict__ w0, const T* __restrict__ w1, long w_stride,
                                                               const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
-                                                              int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+                                                              int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K, GateAct act) {
   constexpr int WC = 4 / WR;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -291,7 +334,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
         const int c = n0 + ct * 16 + 4 * j + i;
         if (c >= N) continue;
         float v = acc0[rt][ct][i];
-        if (GATED) v = v / (1.f + expf(-v)) * acc1[rt][ct][i];
+        if (GATED) v = gated_value(v, acc1[rt][ct][i], act);
         if (out_dtype == CWM_F32)
           ((float*)out)[base + c] = v;
         else
@@ -310,7 +353,7 @@ template <typename T, bool GATED>
 __global__ void __launch_bounds__(256) grouped_stream_kernel(const T* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
                                                              const T* __restrict__ w0, const T* __restrict__ w1, long w_stride,
                                                              const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
-                                                             int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+                                                             int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K, GateAct act) {
   __shared__ float sums[4][GATED ? 2 : 1][64][4];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -382,7 +425,7 @@ __global__ void __launch_bounds__(256) grouped_stream_kernel(const T* __restrict
     float v = ((sums[0][0][lane][i] + sums[1][0][lane][i]) + sums[2][0][lane][i]) + sums[3][0][lane][i];
     if (GATED) {
       const float u = ((sums[0][GATED ? 1 : 0][lane][i] + sums[1][GATED ? 1 : 0][lane][i]) + sums[2][GATED ? 1 : 0][lane][i]) + sums[3][GATED ? 1 : 0][lane][i];
-      v = v / (1.f + expf(-v)) * u;
+      v = gated_value(v, u, act);
     }
     if (out_dtype == CWM_F32)
       ((float*)out)[base + c] = v;
@@ -400,7 +443,7 @@ template <bool GATED>
 __global__ void __launch_bounds__(256) grouped_tiled_kernel(const bf16_t* __restrict__ a, long a_ld, long a_batch, const int* __restrict__ row_token,
                                                             const bf16_t* __restrict__ w0, const bf16_t* __restrict__ w1, long w_stride,
                                                             const int* __restrict__ tile_expert, int n_tiles, void* __restrict__ out,
-                                                            int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K) {
+                                                            int out_dtype, long out_ld, long out_batch, int n_rows, int N, int K, GateAct act) {
   extern __shared__ uint4 tiled_lds[];  // [2 buffers][rows: 128 x 8 pieces | weights: 128 x 8 pieces]
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -533,7 +576,7 @@ __global__ void __launch_bounds__(256) grouped_tiled_kernel(const bf16_t* __rest
         const int c = n0 + (GATED ? wc * 32 : wc * 64) + ct * 16 + 4 * j + i;
         if (c >= N) continue;
         float v = acc0[rt][ct][i];
-        if (GATED) v = v / (1.f + expf(-v)) * acc1[rt][ct][i];
+        if (GATED) v = gated_value(v, acc1[rt][ct][i], act);
         if (out_dtype == CWM_F32)
           ((float*)out)[base + c] = v;
         else
@@ -545,26 +588,30 @@ __global__ void __launch_bounds__(256) grouped_tiled_kernel(const bf16_t* __rest
 template <typename T, int RT, int CT, int WR, bool GATED>
 static void launch_grouped(bool vec, int tiles, int n_batch, hipStream_t stream, const T* a, long a_ld, long a_batch, const int* row_token,
                            const T* w0, const T* w1, long w_stride, const int* tile_expert, int n_tiles, void* out, int out_dtype,
-                           long out_ld, long out_batch, int n_rows, int N, int K) {
+                           long out_ld, long out_batch, int n_rows, int N, int K, GateAct act) {
   constexpr int block_tiles = WR * RT, block_cols = (4 / WR) * CT * 16;
   dim3 grid((tiles + block_tiles - 1) / block_tiles, (N + block_cols - 1) / block_cols, n_batch);
   if (vec)
     hipLaunchKernelGGL((grouped_product_kernel<T, RT, CT, WR, GATED, true>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1,
-                       w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+                       w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K, act);
   else
     hipLaunchKernelGGL((grouped_product_kernel<T, RT, CT, WR, GATED, false>), grid, dim3(256), 0, stream, a, a_ld, a_batch, row_token, w0, w1,
-                       w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+                       w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K, act);
 }
 
 // a: rows of K values, `a_ld` apart (row `row_token[row]` for list row `row` if a list is given; batch z starts
 // `a_batch` further).  w0 (and w1 for the gated form): [experts or batches][N][K], `w_stride` apart.  With
 // `tile_expert` the rows are the list's n_tiles * 16 and out is [rows][out_ld]; without, every batch z < n_batch
 // multiplies the same n_rows rows by its own weight into out + z * out_batch.  tiles_a_block: 1, 4 or 8 row tiles
-// a block (with a list, an expert's tiles start at a multiple of it).
+// a block (with a list, an expert's tiles start at a multiple of it).  act_kind, act_alpha, act_limit: the gated
+// form's activation (`GateAct`).
 extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int dtype, const int* row_token, const void* w0, const void* w1,
                                    long w_stride, const int* tile_expert, int n_tiles, int n_batch, void* out, int out_dtype, long out_ld,
-                                   long out_batch, int n_rows, int N, int K, int tiles_a_block, hipStream_t stream) {
+                                   long out_batch, int n_rows, int N, int K, int tiles_a_block, int act_kind, float act_alpha,
+                                   float act_limit, hipStream_t stream) {
   CWM_REQUIRE(a && w0 && out, "grouped_product: arguments missing");
+  CWM_REQUIRE(act_kind == 0 || act_kind == 1, "grouped_product: unknown gated activation %d", act_kind);
+  const GateAct act = {act_kind, act_alpha, act_limit};
   CWM_REQUIRE(N > 0 && K > 0 && a_ld >= K && out_ld >= 0, "grouped_product: bad sizes");
   CWM_REQUIRE(tile_expert ? (n_tiles >= 0 && n_batch == 1 && row_token) : (n_batch >= 1 && n_batch <= 65535), "grouped_product: give a tile list or a number of batches");
   const int tiles = tile_expert ? n_tiles : (n_rows + TILE_ROWS - 1) / TILE_ROWS;
@@ -578,7 +625,7 @@ extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int d
   const int nb = tile_expert ? 1 : n_batch;
 #define CWM_GROUPED(T, RT, CT, WR, GATED)                                                                                                 \
   launch_grouped<T, RT, CT, WR, GATED>(vec, tiles, nb, stream, (const T*)a, a_ld, a_batch, row_token, (const T*)w0, (const T*)w1, w_stride, \
-                                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K)
+                                       tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K, act)
 #define CWM_GROUPED_SHAPES(T)                                                   \
   do {                                                                          \
     if (w1) {                                                                   \
@@ -596,7 +643,7 @@ extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int d
     dim3 grid(tiles, (N + 15) / 16, nb);
 #define CWM_STREAMED(T, GATED)                                                                                                             \
   hipLaunchKernelGGL((grouped_stream_kernel<T, GATED>), grid, dim3(256), 0, stream, (const T*)a, a_ld, a_batch, row_token, (const T*)w0,     \
-                     (const T*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K)
+                     (const T*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K, act)
     if (dtype == CWM_BF16) {
       if (w1) CWM_STREAMED(bf16_t, true); else CWM_STREAMED(bf16_t, false);
     } else {
@@ -611,10 +658,10 @@ extern "C" int cwm_grouped_product(const void* a, long a_ld, long a_batch, int d
     dim3 grid((tiles + 7) / 8, w1 ? (N + 63) / 64 : (N + 127) / 128, nb);
     if (w1)
       hipLaunchKernelGGL(grouped_tiled_kernel<true>, grid, dim3(256), lds_bytes, stream, (const bf16_t*)a, a_ld, a_batch, row_token,
-                         (const bf16_t*)w0, (const bf16_t*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+                         (const bf16_t*)w0, (const bf16_t*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K, act);
     else
       hipLaunchKernelGGL(grouped_tiled_kernel<false>, grid, dim3(256), lds_bytes, stream, (const bf16_t*)a, a_ld, a_batch, row_token,
-                         (const bf16_t*)w0, (const bf16_t*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K);
+                         (const bf16_t*)w0, (const bf16_t*)w1, w_stride, tile_expert, n_tiles, out, out_dtype, out_ld, out_batch, n_rows, N, K, act);
     return cwm_launch_status("grouped_product");
   }
   if (dtype == CWM_BF16)

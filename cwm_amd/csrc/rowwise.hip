@@ -370,3 +370,57 @@ extern "C" int cwm_sum_partials(void* out, int out_dtype, const float* partials,
     return cwm_fail("sum_partials: unknown dtype %d", out_dtype);
   return cwm_launch_status("sum_partials");
 }
+
+// ---- out = act(sum over p of x[p]) ------------------------------------------------ //
+// The activation between the two products of a feed-forward without a gate: `x` is [count] values of type TX, or
+// n_partials float32 slabs `count` apart that are added in order first; float32 arithmetic, rounded once.
+// kind 0: the square of relu; 1: relu; 2: gelu (tanh form); 3: silu.
+#define CWM_ACT_KINDS 4
+__device__ __forceinline__ float act_value(float z, int kind) {
+  switch (kind) {
+    case 0: {
+      const float r = fmaxf(z, 0.f);
+      return r * r;
+    }
+    case 1:
+      return fmaxf(z, 0.f);
+    case 2:
+      return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    default:
+      return z / (1.f + expf(-z));
+  }
+}
+
+template <typename TX, typename TO>
+__global__ void act_rows_kernel(TO* __restrict__ out, const TX* __restrict__ x, int n_partials, long count, int kind) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (; i < count; i += stride) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += Elem<TX>::load(x + (size_t)p * count + i);
+    Elem<TO>::store(out + i, act_value(v, kind));
+  }
+}
+
+extern "C" int cwm_act_rows(void* out, int out_dtype, const void* x, int x_dtype, int n_partials, long count, int kind,
+                            hipStream_t stream) {
+  CWM_REQUIRE(n_partials >= 1 && count >= 0, "act_rows: bad sizes");
+  CWM_REQUIRE(n_partials == 1 || x_dtype == CWM_F32, "act_rows: partial sums must be float32");
+  CWM_REQUIRE(kind >= 0 && kind < CWM_ACT_KINDS, "act_rows: unknown activation %d", kind);
+  if (count == 0) return 0;
+  long blocks = (count + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  const int key = (x_dtype << 1) | out_dtype;
+#define CWM_ACT_LAUNCH(TX, TO)                                                                                        \
+  hipLaunchKernelGGL((act_rows_kernel<TX, TO>), dim3((unsigned)blocks), dim3(256), 0, stream, (TO*)out, (const TX*)x, \
+                     n_partials, count, kind)
+  switch (key) {
+    case 0: CWM_ACT_LAUNCH(float, float); break;
+    case 1: CWM_ACT_LAUNCH(float, bf16_t); break;
+    case 2: CWM_ACT_LAUNCH(bf16_t, float); break;
+    case 3: CWM_ACT_LAUNCH(bf16_t, bf16_t); break;
+    default: return cwm_fail("act_rows: unknown dtypes x=%d out=%d", x_dtype, out_dtype);
+  }
+#undef CWM_ACT_LAUNCH
+  return cwm_launch_status("act_rows");
+}

@@ -802,6 +802,11 @@ def rope_kv_write(
     )
 
 
+def _check_sink(sink: Optional[torch.Tensor], n_q: int) -> None:
+    if sink is not None and (sink.dtype != torch.float32 or sink.shape != (n_q,) or not sink.is_contiguous()):
+        raise KernelError(f"the sinks must be a contiguous float32 [{n_q}] tensor, one a query head")
+
+
 def paged_attention_simple(
     q: torch.Tensor,
     cache: torch.Tensor,
@@ -811,13 +816,16 @@ def paged_attention_simple(
     window: Optional[int],
     scale: float,
     max_keys: Optional[int] = None,
+    sink: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal attention of `q` [T, Hq, hd] over the paged cache by the plain kernel:
     float32 arithmetic, a key/value head's query heads sharing its keys and values, long
     key ranges cut into segments that a second kernel joins.  `window`: keys read per
     query, own included (None: all).  `max_keys`: the most keys any token reads (default:
-    from the largest position, which costs a copy to the host).  Returns [T, Hq * hd]."""
-    _need_gpu(q, cache, block_table, positions, seq_of_token)
+    from the largest position, which costs a copy to the host).  `sink`: float32 [Hq], a term exp(sink) that
+    each head's softmax denominator holds beside its keys (no key, no value, not scaled).  Returns [T, Hq * hd]."""
+    _need_gpu(q, cache, block_table, positions, seq_of_token, sink)
+    _check_sink(sink, q.shape[1] if q.dim() == 3 else 0)
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
         raise KernelError("q must be [T, Hq, hd] with contiguous heads")
     n_tokens, n_q, hd = q.shape
@@ -851,7 +859,7 @@ def paged_attention_simple(
             _ptr(positions), _ptr(seq_of_token), ctypes.c_int(n_tokens), ctypes.c_int(n_q), ctypes.c_int(n_kv),
             ctypes.c_int(hd), ctypes.c_int(cache.shape[3] // hd), ctypes.c_int(cache.shape[0]),
             ctypes.c_int(-1 if window is None else window - 1), ctypes.c_float(scale),
-            ctypes.c_int(max_keys), _ptr(partial), _stream(),
+            ctypes.c_int(max_keys), _ptr(partial), _ptr(sink), _stream(),
         ),
     )
     return out
@@ -987,10 +995,12 @@ def paged_attention_mfma(
     batch,
     window: Optional[int],
     scale: float,
+    sink: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Matrix-core attention (bfloat16): prompt portions and decoded tokens in one
-    launch, long key ranges of short sequences split and merged."""
-    _need_gpu(q, cache, block_table)
+    launch, long key ranges of short sequences split and merged.  `sink`: as in `paged_attention_simple`."""
+    _need_gpu(q, cache, block_table, sink)
+    _check_sink(sink, q.shape[1] if q.dim() == 3 else 0)
     if q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16:
         raise KernelError("the matrix-core attention kernel takes bfloat16 only")
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
@@ -1028,7 +1038,7 @@ def paged_attention_mfma(
             _ptr(plan.merge), ctypes.c_int(plan.n_merge), ctypes.c_int(plan.n_merge_mid), ctypes.c_int(plan.n_merge_wide), _ptr(partial),
             ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(hd), ctypes.c_int(page_size),
             ctypes.c_int(cache.shape[0]), ctypes.c_int(-1 if window is None else window - 1),
-            ctypes.c_float(scale), _stream(),
+            ctypes.c_float(scale), _ptr(sink), _stream(),
         ),
     )
     return out
@@ -1041,6 +1051,7 @@ def paged_attention(
     batch,
     window: Optional[int],
     scale: float,
+    sink: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Attention of the step's tokens over the cache.  `batch` is the step's
     `StepBatch` (positions, sequence of each token and the per-sequence lengths).
@@ -1048,10 +1059,10 @@ def paged_attention(
     matrix cores; float32, and other sizes, on the plain kernel."""
     hd = q.shape[2]
     if q.is_cuda and mfma_attention_takes(q.dtype, hd, cache.shape[3] // hd):
-        return paged_attention_mfma(q, cache, block_table, batch, window, scale)
+        return paged_attention_mfma(q, cache, block_table, batch, window, scale, sink)
     static = getattr(batch, "static", None)
     max_keys = batch.max_kv_len if static is None else static.max_keys
-    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=max_keys)
+    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=max_keys, sink=sink)
 
 
 # --------------------------------------------------------------------------- #
@@ -1205,6 +1216,7 @@ from .sequence import (  # noqa: E402
     scan_state_unpack, selective_scan, sigmoid_mul, token_shift,
 )
 from .routed import (  # noqa: E402
-    MAX_EXPERTS, MAX_ROUTE_TOP, ExpertGroups, absorb_queries, combine_routed, expand_values, group_by_expert, grouped_gate_up,
-    grouped_linear, route_top,
+    MAX_EXPERTS, MAX_ROUTE_TOP, ExpertGroups, GatedActivation, absorb_queries, combine_routed, expand_values, group_by_expert,
+    grouped_gate_up, grouped_linear, route_top,
 )
+from .streams import ACTIVATIONS, MAX_STREAMS, act_rows, embedding_streams, qk_norm_rope_write, stream_mix_norm  # noqa: E402

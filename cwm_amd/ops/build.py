@@ -58,6 +58,7 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "groupnorm": ({},),
     "state_space": ({},),
     "routed": ({},),
+    "streams": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),
 }
 

@@ -24,11 +24,24 @@ def _base():
     return KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream
 
 
-def route_top(logits: torch.Tensor, top: int) -> Tuple[torch.Tensor, torch.Tensor]:
-    """float32 router logits [T, E] -> (chosen int32 [T, top], weights float32 [T, top]): the `top` largest in
-    falling order (the lower index first among equals) and the softmax over those alone."""
+def route_top(
+    logits: torch.Tensor, top: int, scores: str = "softmax_chosen", correction: Optional[torch.Tensor] = None, scale: float = 1.0,
+    renormalize: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """float32 router logits [T, E] -> (chosen int32 [T, top], weights float32 [T, top]), the chosen in falling order
+    of what they were chosen by (the lower index first among equals).
+    `scores` "softmax_chosen": the `top` largest logits, weighted by the softmax over those alone.
+    `scores` "softmax_all": s = softmax over all experts; the `top` largest of s + `correction` (float32 [E], None for
+    none) are chosen; their weights are `scale` * s (the correction is no part of a weight), divided by the sum of
+    the chosen s first if `renormalize`."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
-    _need_gpu(logits)
+    _need_gpu(logits, correction)
+    if scores not in ("softmax_chosen", "softmax_all"):
+        raise KernelError(f"router scores {scores!r}: 'softmax_chosen' and 'softmax_all' are known")
+    if scores == "softmax_chosen" and (correction is not None or scale != 1.0 or renormalize):
+        raise KernelError("a correction, a scale and renormalised weights belong to router scores over all experts")
+    if correction is not None and (correction.dtype != torch.float32 or correction.shape != (logits.shape[-1],) or not correction.is_contiguous()):
+        raise KernelError("the router's correction must be a contiguous float32 tensor, one value an expert")
     if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
         raise KernelError("router logits must be a contiguous float32 [T, E] tensor")
     n, e = logits.shape
@@ -37,7 +50,13 @@ def route_top(logits: torch.Tensor, top: int) -> Tuple[torch.Tensor, torch.Tenso
     chosen = torch.empty((n, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=logits.device)
     lib = _build.load("routed")
-    _check(lib, lib.cwm_route_top(_ptr(logits), _ptr(chosen), _ptr(weights), ctypes.c_int(n), ctypes.c_int(e), ctypes.c_int(top), _stream()))
+    _check(
+        lib,
+        lib.cwm_route_top(
+            _ptr(logits), _ptr(chosen), _ptr(weights), ctypes.c_int(n), ctypes.c_int(e), ctypes.c_int(top),
+            ctypes.c_int(int(scores == "softmax_all")), _ptr(correction), ctypes.c_float(scale), ctypes.c_int(int(renormalize)), _stream(),
+        ),
+    )
     return chosen, weights
 
 
@@ -88,6 +107,7 @@ def group_by_expert(chosen: torch.Tensor, n_experts: int) -> ExpertGroups:
 def _grouped(
     a: torch.Tensor, a_ld: int, a_batch: int, groups: Optional[ExpertGroups], w0: torch.Tensor, w1: Optional[torch.Tensor],
     out: torch.Tensor, out_ld: int, out_batch: int, n_rows: int, n_batch: int, tiles_a_block: int,
+    activation: Optional["GatedActivation"] = None,
 ) -> None:
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
     _need_gpu(a, w0, w1, out)
@@ -102,19 +122,41 @@ def _grouped(
             _ptr(groups.row_token if groups is not None else None), _ptr(w0), _ptr(w1), ctypes.c_long(n * k),
             _ptr(groups.tile_expert if groups is not None else None), ctypes.c_int(groups.n_tiles if groups is not None else 0),
             ctypes.c_int(n_batch), _ptr(out), ctypes.c_int(_code(out.dtype)), ctypes.c_long(out_ld), ctypes.c_long(out_batch),
-            ctypes.c_int(n_rows), ctypes.c_int(n), ctypes.c_int(k), ctypes.c_int(tiles_a_block), _stream(),
+            ctypes.c_int(n_rows), ctypes.c_int(n), ctypes.c_int(k), ctypes.c_int(tiles_a_block),
+            ctypes.c_int(activation.code() if activation is not None else 0), ctypes.c_float(activation.alpha if activation is not None else 1.0),
+            ctypes.c_float(activation.limit if activation is not None else 0.0), _stream(),
         ),
     )
 
 
-def grouped_gate_up(x: torch.Tensor, groups: ExpertGroups, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """silu(W_gate,e x_t) * (W_up,e x_t) for every pair's row: `x` [T, D] contiguous, weights [E, F, D]; returns
-    [rows, F] in the type of `x` (rows of the padding are not written)."""
+@dataclass(frozen=True)
+class GatedActivation:
+    """What a gated feed-forward makes of g = W_gate x and u = W_up x.
+    "silu": silu(g) * u.
+    "clamped_swish": g' * sigmoid(alpha * g') * (u' + 1) with g' = min(g, limit) and u' = clamp(u, -limit, limit)."""
+
+    kind: str = "silu"
+    alpha: float = 1.0
+    limit: float = 0.0
+
+    def code(self) -> int:
+        kinds = {"silu": 0, "clamped_swish": 1}
+        if self.kind not in kinds:
+            raise ValueError(f"gated activation {self.kind!r}: known are {', '.join(kinds)}")
+        return kinds[self.kind]
+
+
+def grouped_gate_up(
+    x: torch.Tensor, groups: ExpertGroups, gate: torch.Tensor, up: torch.Tensor, activation: Optional[GatedActivation] = None
+) -> torch.Tensor:
+    """act(W_gate,e x_t, W_up,e x_t) for every pair's row, act = silu(g) * u unless `activation` says otherwise:
+    `x` [T, D] contiguous, weights [E, F, D]; returns [rows, F] in the type of `x` (rows of the padding are not
+    written)."""
     KernelError = _base()[0]
     if x.dim() != 2 or not x.is_contiguous() or gate.shape[2] != x.shape[1]:
         raise KernelError("x must be a contiguous [T, D] tensor that fits the experts' weights")
     out = torch.empty((groups.n_tiles * TILE_ROWS, gate.shape[1]), dtype=x.dtype, device=x.device)
-    _grouped(x, x.shape[1], 0, groups, gate, up, out, gate.shape[1], 0, groups.n_tiles * TILE_ROWS, 1, groups.tiles_a_block)
+    _grouped(x, x.shape[1], 0, groups, gate, up, out, gate.shape[1], 0, groups.n_tiles * TILE_ROWS, 1, groups.tiles_a_block, activation)
     return out
 
 

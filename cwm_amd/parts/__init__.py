@@ -1,5 +1,6 @@
 from .base import (
     BLOCKS,
+    CONNECTIONS,
     EMBEDDINGS,
     FEED_FORWARDS,
     HEADS,
@@ -8,6 +9,7 @@ from .base import (
     POSITION_ENCODINGS,
     Block,
     CacheSpec,
+    Connection,
     Embedding,
     FeedForward,
     Head,
@@ -26,13 +28,14 @@ from .base import (
     TensorSpec,
     register_part,
 )
-from . import norm, rope, attention, feedforward, block, embedding, token_shift, state_space, latent_attention, experts  # noqa: F401  (fill the registries)
+from . import norm, rope, attention, feedforward, block, embedding, token_shift, state_space, latent_attention, experts, connection  # noqa: F401  (fill the registries)
 from .linear import LinearWeights
-from .norm import GroupRMSNorm, RMSNorm
+from .norm import GroupRMSNorm, RMSNorm, StreamRMSNorm, StreamUpdate
 from .rope import NoPositionEncoding, RotaryEncoding, llama3_scale_frequencies, rotary_inverse_frequencies
-from .attention import PagedAttention
-from .feedforward import SwiGLU
-from .block import PostNormBlock, PreNormBlock
+from .attention import PagedAttention, SinkAttention
+from .feedforward import ActivatedMLP, SwiGLU
+from .block import ConnectedPreNormBlock, PostNormBlock, PreNormBlock
+from .connection import HyperConnection, ResidualSum
 from .embedding import LinearHead, NormedTokenEmbedding, TokenEmbedding
 from .token_shift import TokenShift
 from .state_space import SelectiveStateSpace

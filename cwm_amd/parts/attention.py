@@ -149,3 +149,115 @@ class PagedAttention(Mixer):
 
 
 register_part("mixer", "paged_attention", PagedAttention)
+
+
+class SinkAttention(Mixer):
+    """Grouped-query attention over a paged cache with a norm over the whole query and key projections, a softmax
+    that holds a learned sink per head, and heads whose values may have another size than their queries and keys.
+
+        q = W_q x, k = W_k x, v = W_v x                          no biases; `n_heads` heads of `qk_dim`, `n_kv_heads` of
+                                                                 `qk_dim` (keys) and `v_dim` (values)
+        q <- q / sqrt(mean(q^2) + eps) * w_q                     over all heads of the projection at once, before the
+        k <- k / sqrt(mean(k^2) + eps) * w_k                     rotation (`qk_norm`; float32)
+        rotation of q and k by the position encoding             its table may rotate fewer than qk_dim dimensions
+        p_j = exp(scale * q . k_j) / (sum_i exp(scale * q . k_i) + exp(sink_h))   over the `window` keys up to the query's own
+        out = W_o [sum_j p_j v_j of every head]
+
+    The sink has no key and no value, is not scaled and counts once.  Keys and values are cached with one head size,
+    the larger of qk_dim and v_dim rounded up to a multiple of 16 (zeros beyond a head's own size, which add nothing to a
+    score and give output columns that W_o, widened by zero columns at load, ignores), so the attention kernels
+    of equal key and value heads serve it.  `names` gives the tensors' local names for the roles q, k, v, o, q_norm,
+    k_norm and sink."""
+
+    replayable = True
+    DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm", "sink": "sink"}
+
+    def __init__(
+        self,
+        dim: int,
+        n_heads: int,
+        n_kv_heads: int,
+        qk_dim: int,
+        v_dim: int,
+        scale: float,
+        window: Optional[int] = None,
+        qk_norm: bool = True,
+        eps: float = 1e-6,
+        sink: bool = True,
+        position_encoding: Optional[PartChoice] = None,
+        names: Optional[Mapping[str, str]] = None,
+    ) -> None:
+        if n_heads % n_kv_heads != 0:
+            raise ValueError(f"{n_heads} query heads do not divide into {n_kv_heads} key/value heads")
+        head_dim = -(-max(qk_dim, v_dim) // 16) * 16
+        if min(qk_dim, v_dim) < 1 or head_dim > MAX_HEAD_DIM:
+            raise ValueError(f"heads of {qk_dim} (queries, keys) and {v_dim} (values) are outside 1..{MAX_HEAD_DIM}, the sizes the attention kernels take")
+        if window is not None and window < 1:
+            raise ValueError("a window holds at least the query's own key")
+        self.dim, self.n_heads, self.n_kv_heads = dim, n_heads, n_kv_heads
+        self.qk_dim, self.v_dim, self.head_dim = qk_dim, v_dim, head_dim
+        self.scale, self.window, self.qk_norm, self.eps, self.sink = float(scale), window, qk_norm, float(eps), sink
+        self.names = {**self.DEFAULT_NAMES, **dict(names or {})}
+        self.position_encoding: Optional[PositionEncoding] = (
+            position_encoding.build("position_encoding") if position_encoding is not None else None
+        )
+
+    def cache_spec(self) -> PagedKVSpec:
+        return PagedKVSpec(n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n = self.names
+        q_out, k_out, v_out = self.n_heads * self.qk_dim, self.n_kv_heads * self.qk_dim, self.n_kv_heads * self.v_dim
+        specs = {
+            n["q"]: TensorSpec((q_out, self.dim)),
+            n["k"]: TensorSpec((k_out, self.dim)),
+            n["v"]: TensorSpec((v_out, self.dim)),
+            n["o"]: TensorSpec((self.dim, self.n_heads * self.v_dim)),
+        }
+        if self.qk_norm:
+            specs[n["q_norm"]] = TensorSpec((q_out,), init="norm", precision="stored")
+            specs[n["k_norm"]] = TensorSpec((k_out,), init="norm", precision="stored")
+        if self.sink:
+            specs[n["sink"]] = TensorSpec((self.n_heads,), init="zeros", precision="stored")
+        return specs
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        n = self.names
+        device = tensors[n["q"]].device
+        self.qkv = LinearWeights.joined([tensors[n["q"]], tensors[n["k"]], tensors[n["v"]]], [None, None, None], stream_copy=runtime.stream_copies)
+        wo = tensors[n["o"]]
+        if self.v_dim != self.head_dim:
+            # the attention kernels return heads of the cached size: columns of zeros where a head's values end
+            wide = torch.zeros((self.dim, self.n_heads, self.head_dim), dtype=wo.dtype, device=device)
+            wide[:, :, : self.v_dim] = wo.reshape(self.dim, self.n_heads, self.v_dim)
+            wo = wide.reshape(self.dim, self.n_heads * self.head_dim)
+        self.wo = LinearWeights(wo, stream_copy=runtime.stream_copies)
+        self.q_weight = tensors[n["q_norm"]].float().contiguous() if self.qk_norm else None
+        self.k_weight = tensors[n["k_norm"]].float().contiguous() if self.qk_norm else None
+        self.sinks = tensors[n["sink"]].float().contiguous() if self.sink else None
+        self.table: Optional[torch.Tensor] = None
+        if self.position_encoding is not None:
+            self.position_encoding.bind({}, runtime)
+            if self.position_encoding.rotary_pairing() != "adjacent":
+                raise ValueError("this mixer rotates adjacent pairs only")
+            table = self.position_encoding.rotary_table()
+            if table is not None:
+                if 2 * table.numel() > self.qk_dim:
+                    raise ValueError(f"{2 * table.numel()} rotated dimensions exceed the head's {self.qk_dim}")
+                # a frequency of 0 leaves its pair alone: the head's other dimensions, and the padding
+                self.table = torch.zeros(self.head_dim // 2, dtype=torch.float32, device=device)
+                self.table[: table.numel()] = table.to(device)
+
+    def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
+        qkv = self.qkv(x, partials_ok=True)
+        q = ops.qk_norm_rope_write(
+            qkv, self.n_heads, self.n_kv_heads, self.qk_dim, self.v_dim, self.head_dim, self.q_weight, self.k_weight, self.eps,
+            batch.positions, self.table, self.runtime.act_dtype,
+            cache.cache if write_cache else None, cache.block_table if write_cache else None, batch.seq_of_token if write_cache else None,
+        )
+        attn = ops.paged_attention(q, cache.cache, cache.block_table, batch, self.window, self.scale, sink=self.sinks)
+        return self.wo(attn, partials_ok=True)  # added into the residual by the next norm
+
+
+register_part("mixer", "sink_attention", SinkAttention)

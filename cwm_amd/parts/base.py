@@ -12,6 +12,7 @@ Kinds of part and their registries (name -> class):
   POSITION_ENCODINGS  what a mixer applies to queries and keys
   BLOCKS              arrangement of the above in one layer
   EMBEDDINGS          token ids (and whatever else of the step) -> the float32 residual stream
+  CONNECTIONS         how a sublayer reads the residual and how its result goes back into it
   HEADS               normalised rows -> float32 logits
 """
 
@@ -30,7 +31,7 @@ import torch
 class TensorSpec:
     shape: Tuple[int, ...]
     kind: str = "float"  # "float" or "int" (integer tables are kept as int32)
-    init: str = "normal"  # how the random-weights writer fills it: "normal" | "norm" | "zeros"
+    init: str = "normal"  # how the random-weights writer fills it: "normal" | "norm" | "zeros" | "ones" | "identity"
     # type a floating tensor is kept in when the model runs in bfloat16: "activation" casts it to
     # bfloat16 whatever it is stored in (matrices: every product then runs on the bfloat16 kernels, as the
     # reference casts every parameter, cwm/model/parallelize_transformer.py:50-59); "stored" keeps a
@@ -206,6 +207,20 @@ class Head(Part):
         raise NotImplementedError
 
 
+class Connection(Part):
+    """How one sublayer is joined to the residual: the coefficients with which it reads the residual's streams
+    (`in_coef()`: float32 [S], None for ones) and what takes its result back (`update(y)`: the pending change that
+    the next norm applies).  The plain sum x <- x + y is the connection of one stream without coefficients."""
+
+    streams = 1
+
+    def in_coef(self) -> Optional[torch.Tensor]:
+        return None
+
+    def update(self, y: torch.Tensor) -> Any:
+        raise NotImplementedError
+
+
 class Block(Part):
     """One layer: an arrangement of any number of norms, mixers and feed-forwards.
 
@@ -281,6 +296,7 @@ POSITION_ENCODINGS: Dict[str, Callable[..., PositionEncoding]] = {}
 BLOCKS: Dict[str, Callable[..., Block]] = {}
 EMBEDDINGS: Dict[str, Callable[..., Embedding]] = {}
 HEADS: Dict[str, Callable[..., Head]] = {}
+CONNECTIONS: Dict[str, Callable[..., Connection]] = {}
 
 _REGISTRIES = {
     "norm": NORMS,
@@ -290,12 +306,13 @@ _REGISTRIES = {
     "block": BLOCKS,
     "embedding": EMBEDDINGS,
     "head": HEADS,
+    "connection": CONNECTIONS,
 }
 
 
 def register_part(kind: str, name: str, factory: Callable[..., Part]) -> None:
     """Make `factory` available to architecture builders as part `name` of `kind`
-    ("norm", "mixer", "feed_forward", "position_encoding", "block", "embedding" or "head")."""
+    ("norm", "mixer", "feed_forward", "position_encoding", "block", "embedding", "head" or "connection")."""
     if kind not in _REGISTRIES:
         raise KeyError(f"unknown kind of part {kind!r}; kinds: {', '.join(_REGISTRIES)}")
     _REGISTRIES[kind][name] = factory

@@ -6,7 +6,7 @@ from typing import Any, Mapping, Optional
 
 import torch
 
-from .base import Block, FeedForward, Mixer, Norm, register_part
+from .base import Block, Connection, FeedForward, Mixer, Norm, register_part
 
 
 class PreNormBlock(Block):
@@ -77,3 +77,36 @@ class PostNormBlock(Block):
 
 
 register_part("block", "post_norm", PostNormBlock)
+
+
+class ConnectedPreNormBlock(Block):
+    """Pre-norm sublayers joined to the residual by connections of their own: the mixer reads
+    norm1(connection1's view of the residual) and its result goes back through connection1, then the same for the
+    feed-forward with norm2 and connection2 where the layer has one.  The residual may be several streams
+    (`HyperConnection`) or one (`ResidualSum`); the norms (`StreamRMSNorm`) apply the pending change of the sublayer
+    before and read the streams in one kernel, so the block takes the previous layer's pending change and returns
+    its own, like `PreNormBlock`."""
+
+    def __init__(
+        self, names: Mapping[str, str], norm1: Norm, connection1: Connection, mixer: Mixer,
+        norm2: Optional[Norm] = None, connection2: Optional[Connection] = None, feed_forward: Optional[FeedForward] = None,
+    ) -> None:
+        if not ((feed_forward is None) == (norm2 is None) == (connection2 is None)):
+            raise ValueError("a feed-forward comes with its norm and its connection")
+        parts = dict(norm1=norm1, connection1=connection1, mixer=mixer)
+        if feed_forward is not None:
+            parts.update(norm2=norm2, connection2=connection2, feed_forward=feed_forward)
+        super().__init__(names, **parts)
+        self.norm1, self.connection1, self.mixer = norm1, connection1, mixer
+        self.norm2, self.connection2, self.feed_forward = norm2, connection2, feed_forward
+
+    def forward(self, h: torch.Tensor, delta: Any, batch: Any, cache: Any, write_cache: bool = True) -> Any:
+        x = self.norm1.forward(h, delta, in_coef=self.connection1.in_coef())
+        delta = self.connection1.update(self.mixer.forward(x, batch, cache, write_cache))
+        if self.feed_forward is not None:
+            x = self.norm2.forward(h, delta, in_coef=self.connection2.in_coef())
+            delta = self.connection2.update(self.feed_forward.forward(x, batch))
+        return delta
+
+
+register_part("block", "connected_pre_norm", ConnectedPreNormBlock)

@@ -17,12 +17,14 @@ class TokenEmbedding(Embedding):
 
     replayable = True
 
-    def __init__(self, vocab_size: int, dim: int, scale: Optional[float] = None, tensor: str = "weight") -> None:
-        """`tensor`: the table's local name ("" where the folder names it by the part's prefix alone)."""
+    def __init__(self, vocab_size: int, dim: int, scale: Optional[float] = None, tensor: str = "weight", streams: int = 1) -> None:
+        """`tensor`: the table's local name ("" where the folder names it by the part's prefix alone).  `streams`: a
+        residual of several streams starts with the scaled row in every one of them, [T, streams * D]."""
         self.vocab_size = vocab_size
         self.dim = dim
         self.scale = 1.0 if scale is None else float(scale)
         self.tensor = tensor
+        self.streams = streams
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {self.tensor: TensorSpec((self.vocab_size, self.dim))}
@@ -32,6 +34,8 @@ class TokenEmbedding(Embedding):
         self.table = tensors[self.tensor].contiguous()
 
     def forward(self, batch: Any) -> torch.Tensor:
+        if self.streams > 1:
+            return ops.embedding_streams(batch.tokens, self.table, self.streams, self.scale)
         return ops.embedding(batch.tokens, self.table, self.scale)
 
 

@@ -1,4 +1,4 @@
-"""Dense gated feed-forward."""
+"""Dense feed-forwards: gated, and with a plain activation between two products."""
 
 from __future__ import annotations
 
@@ -50,3 +50,32 @@ class SwiGLU(FeedForward):
 
 
 register_part("feed_forward", "swiglu", SwiGLU)
+
+
+class ActivatedMLP(FeedForward):
+    """W_down act(W_up x), no gate and no biases; `activation` is one of `ops.ACTIVATIONS` ("relu2": the square of
+    relu).  The activation is computed in float32 on the product's sums and rounded once.  `up` and `down` are
+    the tensors' local names."""
+
+    replayable = True
+
+    def __init__(self, dim: int, hidden_dim: int, activation: str = "relu2", up: str = "up", down: str = "down") -> None:
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r}: known are {', '.join(ops.ACTIVATIONS)}")
+        self.dim, self.hidden_dim, self.activation = dim, hidden_dim, activation
+        self.up_name, self.down_name = up, down
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.up_name: TensorSpec((self.hidden_dim, self.dim)), self.down_name: TensorSpec((self.dim, self.hidden_dim))}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.up = LinearWeights(tensors[self.up_name], stream_copy=runtime.stream_copies)
+        self.down = LinearWeights(tensors[self.down_name], stream_copy=runtime.stream_copies)
+
+    def forward(self, x: torch.Tensor, batch: Any) -> torch.Tensor:
+        hidden = ops.act_rows(self.up(x, partials_ok=True), self.activation, x.dtype)
+        return self.down(hidden, partials_ok=True)
+
+
+register_part("feed_forward", "activated_mlp", ActivatedMLP)

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+from dataclasses import dataclass
 from typing import Dict, Mapping, Optional
 
 import torch
@@ -18,16 +19,22 @@ class RMSNorm(Norm):
 
     replayable = True
 
-    def __init__(self, dim: int, eps: float) -> None:
+    def __init__(self, dim: int, eps: float, offset: float = 0.0, tensor: str = "weight") -> None:
+        """`offset` is added to the stored weight (1 for a weight that is stored around zero and applied as
+        1 + w); `tensor` is the weight's local name ("" where the folder names it by the part's prefix alone)."""
         self.dim = dim
         self.eps = float(eps)
+        self.offset = float(offset)
+        self.tensor = tensor
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.dim,), init="norm", precision="stored")}
+        return {self.tensor: TensorSpec((self.dim,), init="norm" if self.offset == 0.0 else "normal", precision="stored")}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.tensor]
+        if self.offset != 0.0:
+            self.weight = (self.weight.float() + self.offset).contiguous()  # the sum in float32, once
 
     def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.add_rmsnorm(h, delta, self.weight, self.eps, self.runtime.act_dtype, rows)
@@ -89,3 +96,41 @@ class GroupRMSNorm(Norm):
 
 
 register_part("norm", "group_rmsnorm", GroupRMSNorm)
+
+
+@dataclass
+class StreamUpdate:
+    """A sublayer's result that has not yet gone into a residual of several streams: `y` ([T, D] or float32 partial
+    sums [P, T, D]) with the coefficients that take it there, x_t <- sum_s mix[s, t] x_s + out_coef[t] y (float32
+    [S, S] and [S]; None for the identity and ones, which is the plain residual sum)."""
+
+    y: torch.Tensor
+    mix: Optional[torch.Tensor] = None
+    out_coef: Optional[torch.Tensor] = None
+
+
+class StreamRMSNorm(RMSNorm):
+    """RMSNorm of what a sublayer reads from a residual of `streams` vectors a token (float32 [T, streams * D]):
+    u = sum_s in_coef[s] x_s, then u / sqrt(mean(u^2) + eps) * (offset + weight).  The pending `StreamUpdate` of the
+    sublayer before is applied to the streams first, in the same kernel and in float32.  Without `in_coef` every
+    stream counts once: the sum of the streams, which is what a model's final norm reads.  One stream with no
+    coefficients is the ordinary residual."""
+
+    def __init__(self, dim: int, eps: float, streams: int = 1, offset: float = 0.0, tensor: str = "weight") -> None:
+        super().__init__(dim, eps, offset, tensor)
+        if not 1 <= streams <= ops.MAX_STREAMS:
+            raise ValueError(f"{streams} streams: the kernels take 1..{ops.MAX_STREAMS}")
+        self.streams = streams
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.weight = self.weight.float().contiguous()
+
+    def forward(  # type: ignore[override]
+        self, h: torch.Tensor, delta: Optional[StreamUpdate], rows: Optional[torch.Tensor] = None, in_coef: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        y, mix, out_coef = (delta.y, delta.mix, delta.out_coef) if delta is not None else (None, None, None)
+        return ops.stream_mix_norm(h, self.streams, y, mix, out_coef, in_coef, self.weight, self.eps, self.runtime.act_dtype, rows)
+
+
+register_part("norm", "stream_rmsnorm", StreamRMSNorm)

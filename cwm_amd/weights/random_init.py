@@ -49,6 +49,10 @@ def random_tensor(
             raise ValueError(f"norm_init must be 'ones' or 'uniform', found {norm_init!r}")
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
+    elif spec.init == "ones":
+        t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+    elif spec.init == "identity":
+        t = torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=device)
     else:
         t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * std
     return t.to(dtype)

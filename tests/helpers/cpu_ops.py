@@ -103,7 +103,7 @@ def qkv_rope_write(x, weight, bias, n_q_heads, n_kv_heads, head_dim, positions, 
     return qkv
 
 
-def paged_attention(q, cache, block_table, batch, window, scale):
+def paged_attention(q, cache, block_table, batch, window, scale, sink=None):
     n_tokens, n_q, hd = q.shape
     n_kv = cache.shape[2]
     page_size = cache.shape[3] // hd
@@ -126,7 +126,10 @@ def paged_attention(q, cache, block_table, batch, window, scale):
         for h in range(n_q):
             g = h // group
             s = (kk[g] @ q[t, h].float()) * scale
-            w = torch.softmax(s, -1)
+            if sink is not None:  # one more term of the denominator, without a key or a value
+                w = torch.softmax(torch.cat([s, sink[h].float().reshape(1)]), -1)[:-1]
+            else:
+                w = torch.softmax(s, -1)
             out[t, h] = w @ vv[g]
     return out.reshape(n_tokens, n_q * hd).to(q.dtype)
 
@@ -253,7 +256,15 @@ def selective_scan(xbc, dt, dt_bias, a_log, d_skip, state, batch, heads, head_di
     return y
 
 
-def route_top(logits, top):
+def route_top(logits, top, scores="softmax_chosen", correction=None, scale=1.0, renormalize=False):
+    if scores == "softmax_all":
+        s = torch.softmax(logits.float(), -1)
+        choice = s + correction.float() if correction is not None else s
+        chosen = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+        w = torch.gather(s, 1, chosen)
+        if renormalize:
+            w = w / w.sum(-1, keepdim=True)
+        return chosen.to(torch.int32), w * scale
     order = torch.sort(logits, dim=-1, descending=True, stable=True)
     values, chosen = order.values[:, :top], order.indices[:, :top]
     return chosen.to(torch.int32), torch.softmax(values, -1)
@@ -263,11 +274,15 @@ def group_by_expert(chosen, n_experts):
     return chosen  # the stand-ins keep one row a pair, in the order of the pairs
 
 
-def grouped_gate_up(x, groups, gate, up):
+def grouped_gate_up(x, groups, gate, up, activation=None):
     e = groups.reshape(-1).long()
     rows = x.float().repeat_interleave(groups.shape[1], 0)
     g = torch.einsum("rd,rfd->rf", rows, gate.float()[e])
     u = torch.einsum("rd,rfd->rf", rows, up.float()[e])
+    if activation is not None and activation.kind == "clamped_swish":
+        g = g.clamp(max=activation.limit)
+        u = u.clamp(-activation.limit, activation.limit)
+        return (g * torch.sigmoid(activation.alpha * g) * (u + 1)).to(x.dtype)
     return (g * torch.sigmoid(g) * u).to(x.dtype)
 
 
@@ -289,7 +304,73 @@ def expand_values(mixed, lead, weight):
     return torch.einsum("thn,hvn->thv", mixed[:, :, lead:].float(), weight.float()).reshape(mixed.shape[0], -1).to(mixed.dtype)
 
 
+def embedding_streams(tokens, table, streams, scale=1.0):
+    return (table[tokens.long()].float() * scale).repeat(1, streams)
+
+
+def stream_mix_norm(x, streams, y, mix, out_coef, in_coef, weight, eps, out_dtype, rows=None):
+    n = x.shape[0]
+    xs = x.view(n, streams, -1)
+    new = xs
+    if y is not None:
+        if y.dim() == 3:
+            y = y.float().sum(0)
+        m = mix if mix is not None else torch.eye(streams)
+        b = out_coef if out_coef is not None else torch.ones(streams)
+        new = torch.einsum("st,nsd->ntd", m.float(), xs) + b.float()[None, :, None] * y.float()[:, None, :]
+        if rows is None:
+            xs.copy_(new)
+    a = in_coef if in_coef is not None else torch.ones(streams)
+    u = (a.float()[None, :, None] * new).sum(1)
+    if rows is not None:
+        u = u[rows.long()]
+    return (u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
+
+
+def act_rows(x, kind, out_dtype):
+    if x.dim() == 3:
+        x = x.sum(0)
+    z = x.float()
+    if kind == "relu2":
+        z = torch.relu(z) ** 2
+    elif kind == "relu":
+        z = torch.relu(z)
+    elif kind == "gelu_tanh":
+        z = torch.nn.functional.gelu(z, approximate="tanh")
+    else:
+        z = z * torch.sigmoid(z)
+    return z.to(out_dtype)
+
+
+def qk_norm_rope_write(qkv, n_q_heads, n_kv_heads, qk_dim, v_dim, head_dim, q_weight, k_weight, eps, positions, inv_freq, out_dtype,
+                       cache=None, block_table=None, seq_of_token=None):
+    if qkv.dim() == 3:
+        qkv = qkv.sum(0)
+    qkv = qkv.float()
+    n = qkv.shape[0]
+    qw, kw = n_q_heads * qk_dim, n_kv_heads * qk_dim
+    q, k, v = qkv[:, :qw], qkv[:, qw : qw + kw], qkv[:, qw + kw :]
+    if q_weight is not None:
+        q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.float()
+    if k_weight is not None:
+        k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.float()
+
+    def padded(t, heads, width):
+        out = torch.zeros((n, heads, head_dim), dtype=torch.float32)
+        out[:, :, :width] = t.reshape(n, heads, width)
+        return out
+
+    q, k, v = padded(q, n_q_heads, qk_dim), padded(k, n_kv_heads, qk_dim), padded(v, n_kv_heads, v_dim)
+    if inv_freq is not None:
+        q, k = _rotate(q, positions, inv_freq), _rotate(k, positions, inv_freq)
+    q, k, v = q.to(out_dtype), k.to(out_dtype), v.to(out_dtype)
+    if cache is not None:
+        rope_kv_write(q.clone(), k, v, positions, None, cache, block_table, seq_of_token)
+    return q
+
+
 STAND_INS = (
+    "embedding_streams", "stream_mix_norm", "act_rows", "qk_norm_rope_write",
     "embedding", "add_rmsnorm", "silu_mul", "gate_up_silu", "linear", "gemm_f32", "gemm_bf16",
     "rope_kv_write", "qkv_rope_write", "paged_attention", "sample", "sample_packed", "token_logprobs",
     "group_rmsnorm", "cast_rows", "token_shift", "sigmoid_mul", "causal_conv_silu", "selective_scan", "route_top",
