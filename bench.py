@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bf16|fp32]
     python bench.py --shape llama8b --serve 64     (requests through the scheduler instead)
+    python bench.py --compare lapevik|segedra      (another design beside the dense decoder of equal size instead)
 
 Default run: the layer sizes of the CWM-32B shape with random weights, a batch of 8
 requests at a context of 32,768 tokens each; a step is one decode step of the whole
@@ -330,15 +331,38 @@ LAPEVIK_SIZES = {
 }
 
 
-def compare_lapevik(args, device):
-    """Prefill and decode of the Lapevik design at sizes like a real model's layers, beside the dense decoder of equal
+def segedra_config(width, layers, heads, kv_heads, window, streams, ff_dense, ff, experts, top, vocab=32768):
+    """A Segedra model of `layers` layers: attention with heads of 128 in every layer, a dense feed-forward in the
+    first and routed experts in the others, `streams` residual streams."""
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": window},
+             "rot": {"base": 500000.0, "dims": 128}}
+    moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top, "scale": 1.0}}
+    dense = {"kind": "dense", "ff": ff_dense}
+    return {
+        "architecture": "Segedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "streams": streams,
+        "layers": [{"type": "attention", "mixer": mixer, "mlp": dense if i == 0 else moe} for i in range(layers)],
+    }
+
+
+# the same two widths; the dense decoder beside it has the same heads and a feed-forward as wide as a token's experts together
+SEGEDRA_SIZES = {
+    "w2048": (dict(width=2048, layers=8, heads=16, kv_heads=8, window=8192, streams=4, ff_dense=4096, ff=1024, experts=16, top=4), 4096),
+    "w4096": (dict(width=4096, layers=8, heads=32, kv_heads=8, window=8192, streams=4, ff_dense=6144, ff=1536, experts=32, top=4), 6144),
+}
+
+COMPARISONS = {"lapevik": (LAPEVIK_SIZES, lapevik_config), "segedra": (SEGEDRA_SIZES, segedra_config)}
+
+
+def compare_designs(args, device):
+    """Prefill and decode of another design at sizes like a real model's layers, beside the dense decoder of equal
     width, depth and active feed-forward width: one JSON line."""
-    out = {"compare": "lapevik", "dtype": args.dtype, "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens, "sizes": {}}
-    names = [args.size] if args.size else list(LAPEVIK_SIZES)
+    out = {"compare": args.compare, "dtype": args.dtype, "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens, "sizes": {}}
+    all_sizes, make_config = COMPARISONS[args.compare]
+    names = [args.size] if args.size else list(all_sizes)
     for name in names:
-        sizes, hidden = LAPEVIK_SIZES[name]
+        sizes, hidden = all_sizes[name]
         row = {}
-        for label, config in (("lapevik", lapevik_config(**sizes)), ("llama3_dense", dense_like(sizes["width"], sizes["layers"], hidden))):
+        for label, config in ((args.compare, make_config(**sizes)), ("llama3_dense", dense_like(sizes["width"], sizes["layers"], hidden))):
             if args.only and label != args.only:
                 continue
             bench = ShapeBench(f"{label} {name}", config, None, args.dtype, args.page, args.graphs, device)
@@ -386,9 +410,9 @@ def main() -> int:
         "through the engine's scheduler (continuous batching, temperature 0.7, top-p 0.95)",
     )
     ap.add_argument("--new", type=int, default=512, help="tokens generated per request with --serve")
-    ap.add_argument("--compare", default=None, choices=["lapevik"], help="instead of the step benchmark: prefill and decode of another design beside the dense decoder of equal size")
+    ap.add_argument("--compare", default=None, choices=sorted(COMPARISONS), help="instead of the step benchmark: prefill and decode of another design beside the dense decoder of equal size")
     ap.add_argument("--size", default=None, choices=sorted(LAPEVIK_SIZES), help="with --compare: one size only")
-    ap.add_argument("--only", default=None, choices=["lapevik", "llama3_dense"], help="with --compare: one of the two models only")
+    ap.add_argument("--only", default=None, choices=sorted(COMPARISONS) + ["llama3_dense"], help="with --compare: one of the two models only")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -398,7 +422,7 @@ def main() -> int:
 
     device = torch.device("cuda:0")
     if args.compare:
-        print(json.dumps(compare_lapevik(args, device)), flush=True)
+        print(json.dumps(compare_designs(args, device)), flush=True)
         return 0
     shape_name, shape = SHAPES[args.shape]
     if args.config:

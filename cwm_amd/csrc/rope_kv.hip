@@ -287,7 +287,34 @@ extern "C" int cwm_rope_kv_write_partials(void* qkv, long qkv_stride, const floa
 // caller).  Queries go to q_out [T][Hq][head_dim], keys and values into the paged cache (layout at the top of
 // this file).  All arithmetic float32; one block a token.
 #define NORM_ROPE_MAX_HEAD 256
-template <typename TS, typename TO>
+
+// four consecutive elements of a row, and of a cached key
+template <typename T> struct Four;
+template <> struct Four<float> {
+  static __device__ __forceinline__ void add(const float* p, float (&v)[4]) {
+    const float4 x = *(const float4*)p;
+    v[0] += x.x, v[1] += x.y, v[2] += x.z, v[3] += x.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Four<bf16_t> {
+  static __device__ __forceinline__ void add(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *(const uint2*)p;
+    v[0] += __uint_as_float(x.x << 16), v[1] += __uint_as_float(x.x & 0xffff0000u);
+    v[2] += __uint_as_float(x.y << 16), v[3] += __uint_as_float(x.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    uint2 x;
+    x.x = pack2_bf16(v[0], v[1]);
+    x.y = pack2_bf16(v[2], v[3]);
+    *(uint2*)p = x;
+  }
+};
+
+// The blocks of a token (gridDim.y of them) share its heads; each works out the token's two root mean squares itself.
+// VEC: every size is a multiple of 4 and every row starts at a multiple of 16 bytes (8 for bfloat16): a thread
+// takes four consecutive elements, two pairs, at a time.
+template <typename TS, typename TO, bool VEC>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_write_kernel(const TS* __restrict__ src, long src_stride, int n_partials, long partial_stride,
                           TO* __restrict__ q_out, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
@@ -296,7 +323,7 @@ qk_norm_rope_write_kernel(const TS* __restrict__ src, long src_stride, int n_par
                           int table_width, int page_size, int num_pages, int n_q_heads, int n_kv_heads, int qk_dim,
                           int v_dim, int head_dim) {
   __shared__ float scratch[16];
-  __shared__ float cs[NORM_ROPE_MAX_HEAD];  // cos, sin of each pair
+  __shared__ __attribute__((aligned(16))) float cs[NORM_ROPE_MAX_HEAD];  // cos, sin of each pair
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = head_dim / 2;
@@ -306,6 +333,10 @@ qk_norm_rope_write_kernel(const TS* __restrict__ src, long src_stride, int n_par
     float v = 0.f;
     for (int p = 0; p < n_partials; ++p) v += Elem<TS>::load(srow + (size_t)p * partial_stride + e);
     return v;
+  };
+  auto value4 = [&](int e, float (&v)[4]) {
+    v[0] = v[1] = v[2] = v[3] = 0.f;
+    for (int p = 0; p < n_partials; ++p) Four<TS>::add(srow + (size_t)p * partial_stride + e, v);
   };
   TO* kdst = nullptr;
   TO* vdst = nullptr;
@@ -329,53 +360,99 @@ qk_norm_rope_write_kernel(const TS* __restrict__ src, long src_stride, int n_par
     cs[2 * i + 1] = s;
   }
   float q_rstd = 1.f, k_rstd = 1.f;
-  if (q_weight) {
-    float ss = 0.f;
-    for (int e = threadIdx.x; e < q_width; e += blockDim.x) {
-      const float v = value(e);
-      ss += v * v;
+  const bool norm_k = k_weight && cache;
+  if (q_weight || norm_k) {
+    // both sums of squares in one pass over [q | k]; each in the order of its own elements
+    float sq = 0.f, sk = 0.f;
+    const int first = q_weight ? 0 : q_width, last = norm_k ? q_width + k_width : q_width;
+    if constexpr (VEC) {
+      for (int e = first + 4 * threadIdx.x; e < last; e += 4 * blockDim.x) {
+        float v[4];
+        value4(e, v);
+        const float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        if (e < q_width) sq += ss; else sk += ss;
+      }
+    } else {
+      for (int e = first + threadIdx.x; e < last; e += blockDim.x) {
+        const float v = value(e);
+        if (e < q_width) sq += v * v; else sk += v * v;
+      }
     }
-    q_rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)q_width + eps);
-  }
-  if (k_weight && cache) {
-    float ss = 0.f;
-    for (int e = threadIdx.x; e < k_width; e += blockDim.x) {
-      const float v = value(q_width + e);
-      ss += v * v;
-    }
-    k_rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)k_width + eps);
+    if (q_weight) q_rstd = 1.0f / sqrtf(block_sum(sq, scratch) / (float)q_width + eps);
+    if (norm_k) k_rstd = 1.0f / sqrtf(block_sum(sk, scratch) / (float)k_width + eps);
   }
   __syncthreads();  // the table of cosines and sines is complete
   const int n_heads = n_q_heads + (cache ? n_kv_heads : 0);
-  for (int e = threadIdx.x; e < n_heads * half; e += blockDim.x) {
-    const int hh = e / half, i = e - hh * half;
-    const bool is_key = hh >= n_q_heads;
-    const int head = is_key ? hh - n_q_heads : hh;
-    const int base = (is_key ? q_width : 0) + head * qk_dim;
-    const float* weight = is_key ? k_weight : q_weight;
-    const float rstd = is_key ? k_rstd : q_rstd;
-    float re = 0.f, im = 0.f;
-    if (2 * i < qk_dim) re = value(base + 2 * i) * (weight ? rstd * weight[head * qk_dim + 2 * i] : 1.f);
-    if (2 * i + 1 < qk_dim) im = value(base + 2 * i + 1) * (weight ? rstd * weight[head * qk_dim + 2 * i + 1] : 1.f);
-    const float c = cs[2 * i], s = cs[2 * i + 1];
-    const float ore = re * c - im * s, oim = im * c + re * s;
-    TO* dst = nullptr;
-    if (!is_key)
-      dst = q_out + ((size_t)t * n_q_heads + head) * head_dim;
-    else if (kdst)
-      dst = kdst + ((size_t)head * page_size + slot) * head_dim;
-    if (dst) {
-      Elem<TO>::store(dst + 2 * i, ore);
-      Elem<TO>::store(dst + 2 * i + 1, oim);
+  // this block's heads
+  const int per_block = (n_heads + gridDim.y - 1) / gridDim.y;
+  const int head_lo = blockIdx.y * per_block, head_hi = min(n_heads, head_lo + per_block);
+  if constexpr (VEC) {
+    const int quarter = head_dim / 4;
+    for (int e = head_lo * quarter + threadIdx.x; e < head_hi * quarter; e += blockDim.x) {
+      const int hh = e / quarter, d0 = 4 * (e - hh * quarter);
+      const bool is_key = hh >= n_q_heads;
+      const int head = is_key ? hh - n_q_heads : hh;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      if (d0 < qk_dim) {
+        value4((is_key ? q_width : 0) + head * qk_dim + d0, v);
+        const float* weight = is_key ? k_weight : q_weight;
+        if (weight) {
+          const float rstd = is_key ? k_rstd : q_rstd;
+          const float4 w = *(const float4*)(weight + head * qk_dim + d0);
+          v[0] *= rstd * w.x, v[1] *= rstd * w.y, v[2] *= rstd * w.z, v[3] *= rstd * w.w;
+        }
+      }
+      const float4 r = *(const float4*)(cs + d0);  // cos, sin of the pair d0 / 2 and of the next
+      const float o[4] = {v[0] * r.x - v[1] * r.y, v[1] * r.x + v[0] * r.y, v[2] * r.z - v[3] * r.w, v[3] * r.z + v[2] * r.w};
+      if (!is_key)
+        Four<TO>::store(q_out + ((size_t)t * n_q_heads + head) * head_dim + d0, o);
+      else if (kdst)
+        Four<TO>::store(kdst + ((size_t)head * page_size + slot) * head_dim + d0, o);
+    }
+  } else {
+    for (int e = head_lo * half + threadIdx.x; e < head_hi * half; e += blockDim.x) {
+      const int hh = e / half, i = e - hh * half;
+      const bool is_key = hh >= n_q_heads;
+      const int head = is_key ? hh - n_q_heads : hh;
+      const int base = (is_key ? q_width : 0) + head * qk_dim;
+      const float* weight = is_key ? k_weight : q_weight;
+      const float rstd = is_key ? k_rstd : q_rstd;
+      float re = 0.f, im = 0.f;
+      if (2 * i < qk_dim) re = value(base + 2 * i) * (weight ? rstd * weight[head * qk_dim + 2 * i] : 1.f);
+      if (2 * i + 1 < qk_dim) im = value(base + 2 * i + 1) * (weight ? rstd * weight[head * qk_dim + 2 * i + 1] : 1.f);
+      const float c = cs[2 * i], s = cs[2 * i + 1];
+      const float ore = re * c - im * s, oim = im * c + re * s;
+      TO* dst = nullptr;
+      if (!is_key)
+        dst = q_out + ((size_t)t * n_q_heads + head) * head_dim;
+      else if (kdst)
+        dst = kdst + ((size_t)head * page_size + slot) * head_dim;
+      if (dst) {
+        Elem<TO>::store(dst + 2 * i, ore);
+        Elem<TO>::store(dst + 2 * i + 1, oim);
+      }
     }
   }
   if (vdst) {
     const int v_block = (page_size % 8 == 0) ? 8 : page_size;
     const int v_base = q_width + k_width;
-    for (int e = threadIdx.x; e < n_kv_heads * head_dim; e += blockDim.x) {
-      const int head = e / head_dim, d = e - head * head_dim;
-      const float v = d < v_dim ? value(v_base + head * v_dim + d) : 0.f;
-      Elem<TO>::store(vdst + (size_t)head * head_dim * page_size + ((size_t)(slot / v_block) * head_dim + d) * v_block + slot % v_block, v);
+    const int first = blockIdx.y * blockDim.x + threadIdx.x, step = gridDim.y * blockDim.x;
+    if constexpr (VEC) {
+      const int quarter = head_dim / 4;
+      for (int e = first; e < n_kv_heads * quarter; e += step) {
+        const int head = e / quarter, d0 = 4 * (e - head * quarter);
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (d0 < v_dim) value4(v_base + head * v_dim + d0, v);
+        TO* dst = vdst + (size_t)head * head_dim * page_size + ((size_t)(slot / v_block) * head_dim + d0) * v_block + slot % v_block;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) Elem<TO>::store(dst + (size_t)i * v_block, v[i]);
+      }
+    } else {
+      for (int e = first; e < n_kv_heads * head_dim; e += step) {
+        const int head = e / head_dim, d = e - head * head_dim;
+        const float v = d < v_dim ? value(v_base + head * v_dim + d) : 0.f;
+        Elem<TO>::store(vdst + (size_t)head * head_dim * page_size + ((size_t)(slot / v_block) * head_dim + d) * v_block + slot % v_block, v);
+      }
     }
   }
 }
@@ -403,10 +480,25 @@ extern "C" int cwm_qk_norm_rope_write(const void* src, int src_dtype, long src_s
   }
   if (n_tokens == 0) return 0;
   const int key = (src_dtype << 1) | out_dtype;
-#define CWM_NORM_ROPE(TS, TO)                                                                                               \
-  hipLaunchKernelGGL((qk_norm_rope_write_kernel<TS, TO>), dim3(n_tokens), dim3(256), 0, stream, (const TS*)src, src_stride, \
-                     n_partials, partial_stride, (TO*)q_out, q_weight, k_weight, eps, positions, seq_of_token, inv_freq,    \
-                     (TO*)cache, block_table, table_width, page_size, num_pages, n_q_heads, n_kv_heads, qk_dim, v_dim, head_dim)
+  const int src_bytes = src_dtype == CWM_F32 ? 4 : 2, out_bytes = out_dtype == CWM_F32 ? 4 : 2;
+  const bool vec = qk_dim % 4 == 0 && v_dim % 4 == 0 && head_dim % 4 == 0 && src_stride % 4 == 0 && partial_stride % 4 == 0 &&
+                   ((uintptr_t)src % (4 * src_bytes)) == 0 && ((uintptr_t)q_out % (4 * out_bytes)) == 0 &&
+                   ((uintptr_t)cache % (4 * out_bytes)) == 0 && ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0;
+  // few tokens: several blocks a token, so that a decode step's rows are not left to as many blocks
+  const int heads = n_q_heads + n_kv_heads;
+  const int gy = n_tokens >= 512 ? 1 : (heads < 8 ? heads : 8);
+#define CWM_NORM_ROPE_V(TS, TO, VEC)                                                                                       \
+  hipLaunchKernelGGL((qk_norm_rope_write_kernel<TS, TO, VEC>), dim3(n_tokens, gy), dim3(256), 0, stream, (const TS*)src,    \
+                     src_stride, n_partials, partial_stride, (TO*)q_out, q_weight, k_weight, eps, positions, seq_of_token, \
+                     inv_freq, (TO*)cache, block_table, table_width, page_size, num_pages, n_q_heads, n_kv_heads, qk_dim,  \
+                     v_dim, head_dim)
+#define CWM_NORM_ROPE(TS, TO)          \
+  do {                                 \
+    if (vec)                           \
+      CWM_NORM_ROPE_V(TS, TO, true);   \
+    else                               \
+      CWM_NORM_ROPE_V(TS, TO, false);  \
+  } while (0)
   switch (key) {
     case 0: CWM_NORM_ROPE(float, float); break;
     case 1: CWM_NORM_ROPE(float, bf16_t); break;
@@ -414,5 +506,6 @@ extern "C" int cwm_qk_norm_rope_write(const void* src, int src_dtype, long src_s
     default: return cwm_fail("qk_norm_rope_write: source type %d with cache type %d is not built", src_dtype, out_dtype);
   }
 #undef CWM_NORM_ROPE
+#undef CWM_NORM_ROPE_V
   return cwm_launch_status("qk_norm_rope_write");
 }

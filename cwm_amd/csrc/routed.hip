@@ -32,19 +32,42 @@ extern "C" int cwm_route_tile_rows() { return TILE_ROWS; }
 // mode 0: the `top` largest logits, weights = softmax over those alone.
 // mode 1: scores s = softmax over all experts; the `top` largest of s + correction (correction: null for none) are
 //         chosen; weights = scale * s of the chosen, divided by their sum first if `renormalize`.
+// One wavefront a token: lane l holds the experts l, l + 64, ...; a choice is a vote of the lanes (the larger value, the
+// lower index among equals), so a token's router costs `top` rounds of shuffles whatever the number of experts.
+#define ROUTE_PER_LANE (ROUTE_MAX_EXPERTS / CWM_WAVE)
 __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ chosen,
                                                         float* __restrict__ weights, int n_tokens, int n_experts, int top, int mode,
                                                         const float* __restrict__ correction, float scale, int renormalize) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = threadIdx.x & (CWM_WAVE - 1);
+  const int t = blockIdx.x * (blockDim.x / CWM_WAVE) + threadIdx.x / CWM_WAVE;
   if (t >= n_tokens) return;
   const float* z = logits + (size_t)t * n_experts;
-  float largest_all = 0.f, inv_all = 1.f;
+  const float neg_inf = -__builtin_inff();
+  float score[ROUTE_PER_LANE], choice[ROUTE_PER_LANE];  // what a weight is made of, what an expert is chosen by
+#pragma unroll
+  for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+    const int e = lane + CWM_WAVE * i;
+    score[i] = e < n_experts ? z[e] : neg_inf;
+    choice[i] = score[i];
+  }
   if (mode == 1) {
-    largest_all = z[0];
-    for (int e = 1; e < n_experts; ++e) largest_all = fmaxf(largest_all, z[e]);
-    float sum_all = 0.f;
-    for (int e = 0; e < n_experts; ++e) sum_all += expf(z[e] - largest_all);
-    inv_all = 1.f / sum_all;
+    float largest = score[0];
+#pragma unroll
+    for (int i = 1; i < ROUTE_PER_LANE; ++i) largest = fmaxf(largest, score[i]);
+    largest = wave_max(largest);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+      score[i] = lane + CWM_WAVE * i < n_experts ? expf(score[i] - largest) : 0.f;
+      sum += score[i];
+    }
+    const float inv = 1.f / wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+      const int e = lane + CWM_WAVE * i;
+      score[i] *= inv;
+      choice[i] = e < n_experts ? (correction ? score[i] + correction[e] : score[i]) : neg_inf;
+    }
   }
   int idx[ROUTE_MAX_TOP];
   float val[ROUTE_MAX_TOP];
@@ -56,27 +79,39 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
 #pragma unroll
   for (int k = 0; k < ROUTE_MAX_TOP; ++k) {
     if (k < top) {
-      int best = -1;
-      float bv = 0.f, bs = 0.f;
-      for (int e = 0; e < n_experts; ++e) {
-        bool taken = false;
+      // this lane's best expert that is not taken yet, then the wavefront's
+      float bv = neg_inf, bs = 0.f;
+      int be = 0x7fffffff;
 #pragma unroll
-        for (int m = 0; m < ROUTE_MAX_TOP; ++m) taken |= (m < k && idx[m] == e);
-        float v = z[e], score = v;
-        if (mode == 1) {
-          score = expf(v - largest_all) * inv_all;
-          v = correction ? score + correction[e] : score;
-        }
-        if (!taken && (best < 0 || v > bv)) {
-          best = e;
-          bv = v;
-          bs = score;
+      for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+        const int e = lane + CWM_WAVE * i;
+        if (e < n_experts && (be == 0x7fffffff || choice[i] > bv)) {  // taken experts have left the vote (below)
+          bool taken = false;
+#pragma unroll
+          for (int m = 0; m < ROUTE_MAX_TOP; ++m) taken |= (m < k && idx[m] == e);
+          if (!taken) {
+            bv = choice[i];
+            bs = score[i];
+            be = e;
+          }
         }
       }
-      idx[k] = best;
-      val[k] = mode == 1 ? bs : bv;
+#pragma unroll
+      for (int off = CWM_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, CWM_WAVE), os = __shfl_xor(bs, off, CWM_WAVE);
+        const int oe = __shfl_xor(be, off, CWM_WAVE);
+        const bool theirs = oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be));
+        if (theirs) {
+          bv = ov;
+          bs = os;
+          be = oe;
+        }
+      }
+      idx[k] = be;
+      val[k] = bs;
     }
   }
+  if (lane != 0) return;
   float sum = 0.f;
   if (mode == 0) {
     const float largest = val[0];  // the first chosen is the largest
@@ -105,9 +140,10 @@ extern "C" int cwm_route_top(const float* logits, int* chosen, float* weights, i
   CWM_REQUIRE(logits && chosen && weights, "route_top: arguments missing");
   CWM_REQUIRE(top >= 1 && top <= ROUTE_MAX_TOP && top <= n_experts, "route_top: %d of %d experts, the kernel takes up to %d", top, n_experts,
               ROUTE_MAX_TOP);
+  CWM_REQUIRE(n_experts <= ROUTE_MAX_EXPERTS, "route_top: %d experts, the kernel takes up to %d", n_experts, ROUTE_MAX_EXPERTS);
   CWM_REQUIRE(mode == 0 || mode == 1, "route_top: unknown mode %d", mode);
   if (n_tokens <= 0) return 0;
-  hipLaunchKernelGGL(route_top_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, stream, logits, chosen, weights, n_tokens, n_experts, top,
+  hipLaunchKernelGGL(route_top_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, logits, chosen, weights, n_tokens, n_experts, top,
                      mode, correction, scale, renormalize);
   return cwm_launch_status("route_top");
 }

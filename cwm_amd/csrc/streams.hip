@@ -19,12 +19,37 @@ CWM_DEFINE_ERROR_API
 
 extern "C" int cwm_streams_max() { return STREAMS_MAX; }
 
-template <typename TY, typename TO, int S>
+// four consecutive elements
+template <typename T> struct Four;
+template <> struct Four<float> {
+  static __device__ __forceinline__ void add(const float* p, float (&v)[4]) {
+    const float4 x = *(const float4*)p;
+    v[0] += x.x, v[1] += x.y, v[2] += x.z, v[3] += x.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Four<bf16_t> {
+  static __device__ __forceinline__ void add(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *(const uint2*)p;
+    v[0] += __uint_as_float(x.x << 16), v[1] += __uint_as_float(x.x & 0xffff0000u);
+    v[2] += __uint_as_float(x.y << 16), v[3] += __uint_as_float(x.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    uint2 x;
+    x.x = pack2_bf16(v[0], v[1]);
+    x.y = pack2_bf16(v[2], v[3]);
+    *(uint2*)p = x;
+  }
+};
+
+// W: elements a thread takes at a time (4 where the row's length is a multiple of 4 and every row starts at a
+// multiple of 16 bytes, else 1).  A row's sum of squares is added up in the same order for every W.
+template <typename TY, typename TO, int S, int W>
 __global__ void stream_mix_norm_kernel(float* __restrict__ x, const TY* __restrict__ y, int n_partials, long partial_stride,
                                        const float* __restrict__ mix, const float* __restrict__ out_coef,
                                        const float* __restrict__ in_coef, const float* __restrict__ weight,
                                        TO* __restrict__ out, const int* __restrict__ rows, int dim, float eps) {
-  extern __shared__ float u_row[];  // [dim], then 16 floats of scratch
+  extern __shared__ __attribute__((aligned(16))) float u_row[];  // [dim], then 16 floats of scratch
   float* scratch = u_row + dim;
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
@@ -40,44 +65,86 @@ __global__ void stream_mix_norm_kernel(float* __restrict__ x, const TY* __restri
     for (int t = 0; t < S; ++t) m[s][t] = mix ? mix[s * S + t] : (s == t ? 1.f : 0.f);
   }
   float ss = 0.f;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
-    float xs[S];
+  for (int i = W * threadIdx.x; i < dim; i += W * blockDim.x) {
+    float xs[S][W];
 #pragma unroll
-    for (int s = 0; s < S; ++s) xs[s] = xrow[(size_t)s * dim + i];
-    float u = 0.f;
+    for (int s = 0; s < S; ++s) {
+      if constexpr (W == 4) {
+        const float4 v = *(const float4*)(xrow + (size_t)s * dim + i);
+        xs[s][0] = v.x, xs[s][1] = v.y, xs[s][2] = v.z, xs[s][3] = v.w;
+      } else {
+        xs[s][0] = xrow[(size_t)s * dim + i];
+      }
+    }
+    float u[W];
+#pragma unroll
+    for (int e = 0; e < W; ++e) u[e] = 0.f;
     if (yrow) {
-      float yv = 0.f;
-      for (int p = 0; p < n_partials; ++p) yv += Elem<TY>::load(yrow + (size_t)p * partial_stride + i);
+      float yv[W];
+#pragma unroll
+      for (int e = 0; e < W; ++e) yv[e] = 0.f;
+      for (int p = 0; p < n_partials; ++p) {
+        if constexpr (W == 4)
+          Four<TY>::add(yrow + (size_t)p * partial_stride + i, (float(&)[4])yv);
+        else
+          yv[0] += Elem<TY>::load(yrow + (size_t)p * partial_stride + i);
+      }
 #pragma unroll
       for (int t = 0; t < S; ++t) {
-        float v = 0.f;
+        float v[W];
 #pragma unroll
-        for (int s = 0; s < S; ++s) v += m[s][t] * xs[s];
-        v += b[t] * yv;
-        if (write_back) xrow[(size_t)t * dim + i] = v;
-        u += a[t] * v;
+        for (int e = 0; e < W; ++e) {
+          v[e] = 0.f;
+#pragma unroll
+          for (int s = 0; s < S; ++s) v[e] += m[s][t] * xs[s][e];
+          v[e] += b[t] * yv[e];
+          u[e] += a[t] * v[e];
+        }
+        if (write_back) {
+          if constexpr (W == 4)
+            *(float4*)(xrow + (size_t)t * dim + i) = make_float4(v[0], v[1], v[2], v[3]);
+          else
+            xrow[(size_t)t * dim + i] = v[0];
+        }
       }
     } else {
 #pragma unroll
-      for (int t = 0; t < S; ++t) u += a[t] * xs[t];
+      for (int t = 0; t < S; ++t)
+#pragma unroll
+        for (int e = 0; e < W; ++e) u[e] += a[t] * xs[t][e];
     }
-    u_row[i] = u;
-    ss += u * u;
+#pragma unroll
+    for (int e = 0; e < W; ++e) u_row[i + e] = u[e];
   }
+  __syncthreads();
+  // the sum of squares in one order whatever W was: thread j adds the elements j, j + threads, ...
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) ss += u_row[i] * u_row[i];
   ss = block_sum(ss, scratch);
   const float rstd = 1.0f / sqrtf(ss / (float)dim + eps);
   TO* orow = out + (size_t)r * dim;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) Elem<TO>::store(orow + i, u_row[i] * rstd * weight[i]);
+  if constexpr (W == 4) {
+    for (int i = 4 * threadIdx.x; i < dim; i += 4 * blockDim.x) {
+      const float4 uu = *(const float4*)(u_row + i), ww = *(const float4*)(weight + i);
+      const float o[4] = {uu.x * rstd * ww.x, uu.y * rstd * ww.y, uu.z * rstd * ww.z, uu.w * rstd * ww.w};
+      Four<TO>::store(orow + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) Elem<TO>::store(orow + i, u_row[i] * rstd * weight[i]);
+  }
 }
 
 template <typename TY, typename TO>
-static int launch_stream_mix_norm(int streams, int n_out, int threads, size_t lds, hipStream_t stream, float* x, const void* y,
+static int launch_stream_mix_norm(bool vec, int streams, int n_out, int threads, size_t lds, hipStream_t stream, float* x, const void* y,
                                   int n_partials, long partial_stride, const float* mix, const float* out_coef,
                                   const float* in_coef, const float* weight, void* out, const int* rows, int dim, float eps) {
 #define CWM_STREAMS_CASE(S)                                                                                                  \
   case S:                                                                                                                   \
-    hipLaunchKernelGGL((stream_mix_norm_kernel<TY, TO, S>), dim3(n_out), dim3(threads), lds, stream, x, (const TY*)y,        \
-                       n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps);                 \
+    if (vec)                                                                                                                \
+      hipLaunchKernelGGL((stream_mix_norm_kernel<TY, TO, S, 4>), dim3(n_out), dim3(threads), lds, stream, x, (const TY*)y,   \
+                         n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps);               \
+    else                                                                                                                    \
+      hipLaunchKernelGGL((stream_mix_norm_kernel<TY, TO, S, 1>), dim3(n_out), dim3(threads), lds, stream, x, (const TY*)y,   \
+                         n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps);               \
     break
   switch (streams) {
     CWM_STREAMS_CASE(1);
@@ -111,15 +178,17 @@ extern "C" int cwm_stream_mix_norm(void* x, int streams, const void* y, int y_dt
   CWM_REQUIRE(dim <= 15360, "stream_mix_norm: rows of %d elements do not fit the block's LDS", dim);
   if (n_out == 0) return 0;
   if (!y) y_dtype = CWM_F32;
-  const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
+  const bool vec = dim % 4 == 0 && partial_stride % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+                   ((uintptr_t)weight % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const int threads = dim >= 4096 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
   const size_t lds = ((size_t)dim + 16) * sizeof(float);
   int status;
   const int key = (y_dtype << 1) | out_dtype;
   switch (key) {
-    case 0: status = launch_stream_mix_norm<float, float>(streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
-    case 1: status = launch_stream_mix_norm<float, bf16_t>(streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
-    case 2: status = launch_stream_mix_norm<bf16_t, float>(streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
-    case 3: status = launch_stream_mix_norm<bf16_t, bf16_t>(streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
+    case 0: status = launch_stream_mix_norm<float, float>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
+    case 1: status = launch_stream_mix_norm<float, bf16_t>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
+    case 2: status = launch_stream_mix_norm<bf16_t, float>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
+    case 3: status = launch_stream_mix_norm<bf16_t, bf16_t>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
     default: return cwm_fail("stream_mix_norm: unknown dtypes y=%d out=%d", y_dtype, out_dtype);
   }
   if (status) return status;
