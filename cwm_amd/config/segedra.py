@@ -9,6 +9,7 @@ Strict as every configuration: an unknown key is an error that names it.
 
 from __future__ import annotations
 
+import re
 from dataclasses import dataclass
 from typing import Any, List, Mapping, Optional
 
@@ -123,11 +124,12 @@ class LayerConfig:
         self.mixer_config()  # reject what does not fit now, by key
 
     def mixer_config(self) -> AttentionConfig:
-        if self.type not in MIXER_CONFIGS:
+        kind = re.sub(r"_\d+$", "", self.type)  # a numeric suffix marks another set of sizes of the same mixer
+        if kind not in MIXER_CONFIGS:
             raise ConfigError(f"layer type {self.type!r}: known mixers are {', '.join(sorted(MIXER_CONFIGS))}")
         if not isinstance(self.mixer, Mapping):
             raise ConfigError(f"the sizes of mixer {self.type!r} must be an object")
-        return from_dict(MIXER_CONFIGS[self.type], self.mixer, path="mixer")
+        return from_dict(MIXER_CONFIGS[kind], self.mixer, path="mixer")
 
 
 @dataclass(frozen=True)
