@@ -150,11 +150,12 @@ def read_folder(folder: str):
     return config, load_file(os.path.join(folder, "model.safetensors"))
 
 
-# A router's choice between two experts whose choice scores lie closer than this is not compared in bfloat16: the
-# rounding of the router's input moves a score by about a thousandth, and whichever of the two an implementation then
-# takes is right.  Such tokens are left out (they are few; the float32 comparison leaves none out).
-CLOSE_CALL = 4e-3
-MOST_CLOSE_CALLS = 0.15
+# A router's choice between two experts is not compared in bfloat16 where a change of the router's logits by this
+# share of their size could turn it (see `segedra_plain.route`): what reaches a router in bfloat16 differs from the
+# exact input by about a hundredth after a few layers, and whichever of the two experts an implementation then takes
+# is right.  Such tokens are left out of the bfloat16 comparison; the float32 comparison leaves none out.
+CLOSE_CALL = 0.05
+MOST_CLOSE_CALLS = 0.5
 
 
 class Expected(lapevik.Expected):

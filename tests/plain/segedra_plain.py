@@ -105,13 +105,18 @@ def dense_feed_forward(h: torch.Tensor, t: Mapping[str, torch.Tensor], rounded: 
 
 def route(h: torch.Tensor, t: Mapping[str, torch.Tensor], top: int, scale: float, rounded: bool = False, margins: Optional[list] = None):
     """(chosen [n, top], weights [n, top]): scores over all experts; the correction counts for the choice only.
-    `margins` receives, per token, by how much the last chosen expert's choice score leads the first one left out."""
-    scores = torch.softmax(_bf16(h, rounded) @ t["router"].T, -1)
+    `margins` receives, per token, how clear the choice was: by how much the last chosen expert's choice score leads
+    the first one left out, over how far a relative change of the logits by 1 could move the two scores
+    (d s_e = s_e (d z_e - sum_j s_j d z_j), so at most about (s_a + s_b) * |z|)."""
+    logits = _bf16(h, rounded) @ t["router"].T
+    scores = torch.softmax(logits, -1)
     choice = scores + t["correction"] if "correction" in t else scores
     order = torch.sort(choice, dim=-1, descending=True, stable=True)
     chosen = order.indices[:, :top]
     if margins is not None and top < choice.shape[-1]:
-        margins.append(order.values[:, top - 1] - order.values[:, top])
+        pair = torch.gather(scores, 1, order.indices[:, top - 1 : top + 1]).sum(-1)
+        reach = pair * torch.sqrt((logits * logits).mean(-1)) + 1e-30
+        margins.append((order.values[:, top - 1] - order.values[:, top]) / reach)
     return chosen, torch.gather(scores, 1, chosen) * scale
 
 

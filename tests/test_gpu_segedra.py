@@ -544,3 +544,52 @@ def test_command_line_and_trace_run_as_child_processes(folders, tmp_path):
         want = segedra.expected(folders[name], requests, dtype)
         for rid in requests:
             segedra.check(got[rid], want[rid], dtype, f"trace_run {dtype} {rid}")
+
+
+def random_config(seed: int) -> dict:
+    """A configuration drawn from a seed: every size, count, constant and the order of layers differ from draw to draw."""
+    import random
+
+    rng = random.Random(seed)
+    width = rng.choice([32, 40, 48, 64, 72, 96, 100, 128, 136, 192, 200, 256])
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        kv = rng.choice([1, 2, 3, 4])
+        heads = kv * rng.choice([1, 2, 3, 4])
+        dim = rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 96, 128])
+        vdim = rng.choice([8, 12, 16, 32, 48, 64, 80, 128])
+        rot = (rng.choice([100.0, 10000.0, 250000.0, 1e6]), rng.choice([d for d in (2, 4, 8, 16, 32, 64, 128) if d <= dim] + [dim]))
+        kind = rng.choice(["dense", "moe", "moe", "none"])
+        if kind == "dense":
+            mlp = segedra.dense(rng.choice([20, 36, 64, 100, 256]))
+        elif kind == "moe":
+            experts = rng.randint(2, 12)
+            mlp = segedra.moe(rng.choice([8, 12, 32, 50, 64]), experts, rng.randint(1, experts), rng.choice([0.5, 1.0, 2.0, 7.0]), rng.choice([0.5, 1.0, 2.5]))
+        else:
+            mlp = None
+        window = rng.choice([None, 1, 2, 7, 16, 17, 40, 64, 100])
+        layers.append(segedra.attn(heads, kv, dim, vdim, rng.choice([0.05, 0.1, 0.2]) * (64 / dim) ** 0.5, window=window, rot=rot, mlp=mlp))
+    config = {"architecture": "Segedra", "vocab": rng.randint(50, 700), "width": width, "norm": {"eps": rng.choice([1e-5, 1e-6])},
+              "embedding": {"scale": rng.choice([0.7, 1.0, 1.5]) * width ** 0.5}, "layers": layers}
+    if rng.random() < 0.8:
+        config["streams"] = rng.randint(1, 5)
+    if rng.random() < 0.7:
+        start = rng.randint(0, len(layers) - 1)
+        config["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.randint(1, 3)}
+    return config
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations(tmp_path, seed, dtype):
+    """Other models of the design: whole prompts, and a mixed schedule with pages of another size, against the plain
+    implementation."""
+    config = random_config(seed)
+    folder = segedra.make_folder(tmp_path, f"random{seed}", seed=seed, config=config)
+    vocab = config["vocab"]
+    requests = {f"r{i}": traces.random_tokens(7 * seed + i, n, vocab) for i, n in enumerate([3, 150, 45, 88])}
+    want = segedra.expected(folder, requests, dtype)
+    for steps, page in ((traces.whole(requests), 16), (traces.mixed(requests, max_live=3), 32 if seed % 2 else 8)):
+        got, _, _ = run(folder, dtype, steps, requests, vocab, page_size=page, max_requests=4)
+        for rid in requests:
+            segedra.check(got[rid], want[rid], dtype, f"random configuration {seed} {dtype} {rid}: {json.dumps(config)}")
