@@ -48,13 +48,15 @@ template <typename TY, typename TO, int S, int W>
 __global__ void stream_mix_norm_kernel(float* __restrict__ x, const TY* __restrict__ y, int n_partials, long partial_stride,
                                        const float* __restrict__ mix, const float* __restrict__ out_coef,
                                        const float* __restrict__ in_coef, const float* __restrict__ weight,
-                                       TO* __restrict__ out, const int* __restrict__ rows, int dim, float eps) {
+                                       TO* __restrict__ out, const int* __restrict__ rows, int dim, float eps,
+                                       const int* __restrict__ pair_row, const float* __restrict__ pair_weight, int top) {
   extern __shared__ __attribute__((aligned(16))) float u_row[];  // [dim], then 16 floats of scratch
   float* scratch = u_row + dim;
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xrow = x + (size_t)src * S * dim;
-  const TY* yrow = y ? y + (size_t)src * dim : nullptr;
+  // with pair_row, y holds rows of which the token's result is a weighted sum: sum_k pair_weight[t][k] * y[pair_row[t][k]]
+  const TY* yrow = y ? (pair_row ? y : y + (size_t)src * dim) : nullptr;
   const bool write_back = (y != nullptr) && (rows == nullptr);
   float m[S][S], b[S], a[S];
 #pragma unroll
@@ -83,11 +85,28 @@ __global__ void stream_mix_norm_kernel(float* __restrict__ x, const TY* __restri
       float yv[W];
 #pragma unroll
       for (int e = 0; e < W; ++e) yv[e] = 0.f;
-      for (int p = 0; p < n_partials; ++p) {
-        if constexpr (W == 4)
-          Four<TY>::add(yrow + (size_t)p * partial_stride + i, (float(&)[4])yv);
-        else
-          yv[0] += Elem<TY>::load(yrow + (size_t)p * partial_stride + i);
+      if (pair_row) {
+        for (int k = 0; k < top; ++k) {  // in the order of the token's choices, as the kernel that only adds them up does
+          const int row = pair_row[(size_t)src * top + k];
+          if (row < 0) continue;
+          const float wk = pair_weight[(size_t)src * top + k];
+          float part[W];
+#pragma unroll
+          for (int e = 0; e < W; ++e) part[e] = 0.f;
+          if constexpr (W == 4)
+            Four<TY>::add(yrow + (size_t)row * dim + i, (float(&)[4])part);
+          else
+            part[0] = Elem<TY>::load(yrow + (size_t)row * dim + i);
+#pragma unroll
+          for (int e = 0; e < W; ++e) yv[e] += wk * part[e];
+        }
+      } else {
+        for (int p = 0; p < n_partials; ++p) {
+          if constexpr (W == 4)
+            Four<TY>::add(yrow + (size_t)p * partial_stride + i, (float(&)[4])yv);
+          else
+            yv[0] += Elem<TY>::load(yrow + (size_t)p * partial_stride + i);
+        }
       }
 #pragma unroll
       for (int t = 0; t < S; ++t) {
@@ -136,15 +155,18 @@ __global__ void stream_mix_norm_kernel(float* __restrict__ x, const TY* __restri
 template <typename TY, typename TO>
 static int launch_stream_mix_norm(bool vec, int streams, int n_out, int threads, size_t lds, hipStream_t stream, float* x, const void* y,
                                   int n_partials, long partial_stride, const float* mix, const float* out_coef,
-                                  const float* in_coef, const float* weight, void* out, const int* rows, int dim, float eps) {
+                                  const float* in_coef, const float* weight, void* out, const int* rows, int dim, float eps,
+                                  const int* pair_row, const float* pair_weight, int top) {
 #define CWM_STREAMS_CASE(S)                                                                                                  \
   case S:                                                                                                                   \
     if (vec)                                                                                                                \
       hipLaunchKernelGGL((stream_mix_norm_kernel<TY, TO, S, 4>), dim3(n_out), dim3(threads), lds, stream, x, (const TY*)y,   \
-                         n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps);               \
+                         n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps, pair_row,     \
+                         pair_weight, top);                                                                                  \
     else                                                                                                                    \
       hipLaunchKernelGGL((stream_mix_norm_kernel<TY, TO, S, 1>), dim3(n_out), dim3(threads), lds, stream, x, (const TY*)y,   \
-                         n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps);               \
+                         n_partials, partial_stride, mix, out_coef, in_coef, weight, (TO*)out, rows, dim, eps, pair_row,     \
+                         pair_weight, top);                                                                                  \
     break
   switch (streams) {
     CWM_STREAMS_CASE(1);
@@ -165,16 +187,20 @@ static int launch_stream_mix_norm(bool vec, int streams, int n_out, int threads,
 // x: float32 [n_tokens][streams][dim].  y: null (nothing pending), or [n_tokens][dim] of type y_dtype, or n_partials
 // float32 slabs partial_stride apart.  mix [streams * streams], out_coef [streams], in_coef [streams]: float32, null
 // for the identity / ones.  weight: float32 [dim].  rows: null, or n_out indices of the rows to read (x then stays
-// as it is; what is normalised is still the row after the pending change).
+// as it is; what is normalised is still the row after the pending change).  pair_row (int32 [n_tokens][top], -1: none)
+// and pair_weight (float32 [n_tokens][top]): y is then float32 [any][dim] and token t's pending result is
+// sum_k pair_weight[t][k] * y[pair_row[t][k]], added in the order of k (the weighted sum of a token's experts).
 extern "C" int cwm_stream_mix_norm(void* x, int streams, const void* y, int y_dtype, int n_partials, long partial_stride,
                                    const float* mix, const float* out_coef, const float* in_coef, const float* weight,
                                    void* out, int out_dtype, const int* rows, int n_out, int dim, float eps,
-                                   hipStream_t stream) {
+                                   const int* pair_row, const float* pair_weight, int top, hipStream_t stream) {
   CWM_REQUIRE(n_out >= 0 && dim > 0, "stream_mix_norm: bad sizes rows=%d D=%d", n_out, dim);
   CWM_REQUIRE(streams >= 1 && streams <= STREAMS_MAX, "stream_mix_norm: %d streams, the kernel takes 1..%d", streams, STREAMS_MAX);
   CWM_REQUIRE(n_partials >= 1 && (n_partials == 1 || y_dtype == CWM_F32), "stream_mix_norm: partial sums must be float32");
   CWM_REQUIRE(eps > 0.f, "stream_mix_norm: eps must be positive");
   CWM_REQUIRE(x && weight && out, "stream_mix_norm: arguments missing");
+  CWM_REQUIRE(!pair_row || (y && pair_weight && top >= 1 && y_dtype == CWM_F32 && n_partials == 1),
+              "stream_mix_norm: a weighted sum of rows needs float32 rows, weights and the number of rows a token");
   CWM_REQUIRE(dim <= 15360, "stream_mix_norm: rows of %d elements do not fit the block's LDS", dim);
   if (n_out == 0) return 0;
   if (!y) y_dtype = CWM_F32;
@@ -185,10 +211,10 @@ extern "C" int cwm_stream_mix_norm(void* x, int streams, const void* y, int y_dt
   int status;
   const int key = (y_dtype << 1) | out_dtype;
   switch (key) {
-    case 0: status = launch_stream_mix_norm<float, float>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
-    case 1: status = launch_stream_mix_norm<float, bf16_t>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
-    case 2: status = launch_stream_mix_norm<bf16_t, float>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
-    case 3: status = launch_stream_mix_norm<bf16_t, bf16_t>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps); break;
+    case 0: status = launch_stream_mix_norm<float, float>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps, pair_row, pair_weight, top); break;
+    case 1: status = launch_stream_mix_norm<float, bf16_t>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps, pair_row, pair_weight, top); break;
+    case 2: status = launch_stream_mix_norm<bf16_t, float>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps, pair_row, pair_weight, top); break;
+    case 3: status = launch_stream_mix_norm<bf16_t, bf16_t>(vec, streams, n_out, threads, lds, stream, (float*)x, y, n_partials, partial_stride, mix, out_coef, in_coef, weight, out, rows, dim, eps, pair_row, pair_weight, top); break;
     default: return cwm_fail("stream_mix_norm: unknown dtypes y=%d out=%d", y_dtype, out_dtype);
   }
   if (status) return status;

@@ -1219,4 +1219,4 @@ from .routed import (  # noqa: E402
     MAX_EXPERTS, MAX_ROUTE_TOP, ExpertGroups, GatedActivation, absorb_queries, combine_routed, expand_values, group_by_expert,
     grouped_gate_up, grouped_linear, route_top,
 )
-from .streams import ACTIVATIONS, MAX_STREAMS, act_rows, embedding_streams, qk_norm_rope_write, stream_mix_norm  # noqa: E402
+from .streams import ACTIVATIONS, MAX_STREAMS, RoutedSum, act_rows, embedding_streams, qk_norm_rope_write, stream_mix_norm  # noqa: E402

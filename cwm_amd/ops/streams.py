@@ -6,7 +6,8 @@ the host; there is no CPU path."""
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from dataclasses import dataclass
+from typing import Any, Optional, Union
 
 import torch
 
@@ -20,6 +21,23 @@ def _base():
     from . import KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream  # the shared helpers of this package
 
     return KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream
+
+
+@dataclass
+class RoutedSum:
+    """A token's result as a weighted sum of rows that has not been added up: `rows` float32 [rows, D] as the grouped
+    product leaves them, `groups` the step's pairs grouped by expert (`ExpertGroups`: the row of every (token,
+    choice) pair), `weights` float32 [T, top].  `stream_mix_norm` adds the sum up itself, in the order of a token's
+    choices; `combine()` gives it as a tensor, the same bits."""
+
+    rows: torch.Tensor
+    groups: Any
+    weights: torch.Tensor
+
+    def combine(self) -> torch.Tensor:
+        from . import combine_routed
+
+        return combine_routed(self.rows, self.groups, self.weights)
 
 
 def _coefficients(t: Optional[torch.Tensor], shape: tuple, what: str) -> None:
@@ -53,7 +71,7 @@ def embedding_streams(tokens: torch.Tensor, table: torch.Tensor, streams: int, s
 def stream_mix_norm(
     x: torch.Tensor,
     streams: int,
-    y: Optional[torch.Tensor],
+    y: Union[torch.Tensor, RoutedSum, None],
     mix: Optional[torch.Tensor],
     out_coef: Optional[torch.Tensor],
     in_coef: Optional[torch.Tensor],
@@ -63,12 +81,16 @@ def stream_mix_norm(
     rows: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """`x` is the residual as `streams` vectors a token, float32 [T, streams * D].  If a sublayer's result `y` ([T, D],
-    or float32 partial sums [P, T, D], added in order) is pending, every stream first becomes
+    or float32 partial sums [P, T, D], added in order, or a `RoutedSum`) is pending, every stream first becomes
     x_t <- sum_s mix[s, t] x_s + out_coef[t] y, in place.  Returned, in `out_dtype`: the rows
     u / sqrt(mean(u^2) + eps) * weight with u = sum_t in_coef[t] x_t.  `mix` [S, S], `out_coef` [S], `in_coef` [S]:
     float32, None for the identity and ones.  With `rows` (int32 [R]) only those rows are read and `x` stays as it
     is (what is normalised is still the row after the pending change)."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    routed = None
+    if isinstance(y, RoutedSum):
+        routed, y = y, y.rows
+        _need_gpu(routed.weights, routed.groups.pair_row)
     _need_gpu(x, y, mix, out_coef, in_coef, weight, rows)
     if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous() or streams < 1 or x.shape[1] % streams != 0:
         raise KernelError(f"the residual must be a contiguous float32 [T, {streams} * D] tensor")
@@ -76,7 +98,15 @@ def stream_mix_norm(
         raise KernelError(f"{streams} streams: the kernel takes up to {MAX_STREAMS}")
     n_tokens, dim = x.shape[0], x.shape[1] // streams
     n_partials = 1
-    if y is not None:
+    if routed is not None:
+        top = routed.groups.top
+        if y.dtype != torch.float32 or y.dim() != 2 or y.shape[1] != dim or not y.is_contiguous():
+            raise KernelError(f"the experts' rows must be a contiguous float32 [rows, {dim}] tensor")
+        if routed.weights.dtype != torch.float32 or tuple(routed.weights.shape) != (n_tokens, top) or not routed.weights.is_contiguous():
+            raise KernelError(f"the weights of a weighted sum must be float32 [{n_tokens}, {top}]")
+        if routed.groups.pair_row.numel() != n_tokens * top:
+            raise KernelError("the list of rows does not fit the tokens")
+    elif y is not None:
         if y.dim() == 3:
             if y.dtype != torch.float32:
                 raise KernelError("partial sums must be float32")
@@ -97,7 +127,9 @@ def stream_mix_norm(
         lib.cwm_stream_mix_norm(
             _ptr(x), ctypes.c_int(streams), _ptr(y), ctypes.c_int(_code(y.dtype) if y is not None else 0), ctypes.c_int(n_partials),
             ctypes.c_long(n_tokens * dim), _ptr(mix), _ptr(out_coef), _ptr(in_coef), _ptr(weight), _ptr(out), ctypes.c_int(_code(out_dtype)),
-            _ptr(rows), ctypes.c_int(n_out), ctypes.c_int(dim), ctypes.c_float(eps), _stream(),
+            _ptr(rows), ctypes.c_int(n_out), ctypes.c_int(dim), ctypes.c_float(eps),
+            _ptr(routed.groups.pair_row if routed is not None else None), _ptr(routed.weights if routed is not None else None),
+            ctypes.c_int(routed.groups.top if routed is not None else 0), _stream(),
         ),
     )
     return out

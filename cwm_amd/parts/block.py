@@ -105,7 +105,9 @@ class ConnectedPreNormBlock(Block):
         delta = self.connection1.update(self.mixer.forward(x, batch, cache, write_cache))
         if self.feed_forward is not None:
             x = self.norm2.forward(h, delta, in_coef=self.connection2.in_coef())
-            delta = self.connection2.update(self.feed_forward.forward(x, batch))
+            # a feed-forward whose result is a weighted sum of rows leaves the sum to the norm that reads it next
+            deferred = getattr(self.feed_forward, "forward_deferred", None)
+            delta = self.connection2.update(deferred(x, batch) if deferred is not None else self.feed_forward.forward(x, batch))
         return delta
 
 

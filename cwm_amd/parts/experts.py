@@ -63,6 +63,11 @@ class RoutedExperts(FeedForward):
         self.gate, self.up, self.down = stack("gate"), stack("up"), stack("down")  # [experts, out, in]
 
     def forward(self, x: torch.Tensor, batch: Any) -> torch.Tensor:
+        return self.forward_deferred(x, batch).combine()  # float32 [T, dim]
+
+    def forward_deferred(self, x: torch.Tensor, batch: Any) -> "ops.RoutedSum":
+        """The same without the last kernel: every pair's row and the weights, for a consumer that adds a token's
+        rows up itself (a norm that takes a `RoutedSum` as the pending result)."""
         logits = ops.linear(x, self.router, None, torch.float32)
         if self.scores == "softmax_chosen":
             chosen, weights = ops.route_top(logits, self.top)
@@ -74,7 +79,7 @@ class RoutedExperts(FeedForward):
         else:
             hidden = ops.grouped_gate_up(x, groups, self.gate, self.up, self.activation)
         rows = ops.grouped_linear(hidden, groups, self.down)
-        return ops.combine_routed(rows, groups, weights)  # float32 [T, dim]
+        return ops.RoutedSum(rows, groups, weights)
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

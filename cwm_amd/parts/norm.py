@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Mapping, Optional
+from typing import Any, Dict, Mapping, Optional
 
 import torch
 
@@ -100,11 +100,11 @@ register_part("norm", "group_rmsnorm", GroupRMSNorm)
 
 @dataclass
 class StreamUpdate:
-    """A sublayer's result that has not yet gone into a residual of several streams: `y` ([T, D] or float32 partial
-    sums [P, T, D]) with the coefficients that take it there, x_t <- sum_s mix[s, t] x_s + out_coef[t] y (float32
+    """A sublayer's result that has not yet gone into a residual of several streams: `y` ([T, D], float32 partial
+    sums [P, T, D], or an `ops.RoutedSum`) with the coefficients that take it there, x_t <- sum_s mix[s, t] x_s + out_coef[t] y (float32
     [S, S] and [S]; None for the identity and ones, which is the plain residual sum)."""
 
-    y: torch.Tensor
+    y: Any
     mix: Optional[torch.Tensor] = None
     out_coef: Optional[torch.Tensor] = None
 

@@ -312,6 +312,8 @@ def stream_mix_norm(x, streams, y, mix, out_coef, in_coef, weight, eps, out_dtyp
     n = x.shape[0]
     xs = x.view(n, streams, -1)
     new = xs
+    if y is not None and hasattr(y, "groups"):  # a weighted sum of rows that has not been added up
+        y = combine_routed(y.rows, y.groups, y.weights)
     if y is not None:
         if y.dim() == 3:
             y = y.float().sum(0)

@@ -71,6 +71,30 @@ def test_stream_mix_norm(out_dtype, streams, dim, parts):
     torch.testing.assert_close(xd.cpu().view(n, streams, dim), before.cpu().view(n, streams, dim) + y16.float()[:, None, :], rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("streams,dim", [(4, 128), (1, 50), (3, 72)])
+def test_stream_mix_norm_adds_up_a_weighted_sum_of_rows_itself(streams, dim):
+    """The experts' rows of every (token, choice) pair and the router's weights as the pending result: the same bits as
+    from the rows added up beforehand."""
+    from cwm_amd import ops
+
+    tokens, experts, top = 21, 5, 3
+    g = torch.Generator().manual_seed(2)
+    chosen = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(tokens)]).to(torch.int32)
+    groups = ops.group_by_expert(chosen.to(DEV), experts)
+    rows = rnd((groups.n_tiles * 16, dim), 3).to(DEV)
+    weights = torch.rand((tokens, top), generator=g).to(DEV)
+    routed = ops.RoutedSum(rows, groups, weights)
+    mix, b, a, w = rnd((streams, streams), 3).to(DEV), rnd((streams,), 4).to(DEV), rnd((streams,), 5).to(DEV), (rnd((dim,), 6) + 1).to(DEV)
+    x1 = rnd((tokens, streams * dim), 7).to(DEV)
+    x2 = x1.clone()
+    got = ops.stream_mix_norm(x1, streams, routed, mix, b, a, w, 1e-5, torch.float32)
+    want = ops.stream_mix_norm(x2, streams, routed.combine(), mix, b, a, w, 1e-5, torch.float32)
+    assert torch.equal(got, want) and torch.equal(x1, x2)
+    picked = torch.tensor([20, 4], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.stream_mix_norm(x1, streams, routed, mix, b, a, w, 1e-5, torch.bfloat16, picked),
+                       ops.stream_mix_norm(x2, streams, routed.combine(), mix, b, a, w, 1e-5, torch.bfloat16, picked))
+
+
 def test_embedding_starts_every_stream():
     from cwm_amd import ops
 
@@ -96,7 +120,7 @@ def test_act_rows(dtype, kind):
 
 @pytest.mark.parametrize("src_dtype,dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16)])
 @pytest.mark.parametrize("n_q,n_kv,qk,vd,hd,rot,page_size,norm", [
-    (4, 2, 12, 20, 32, 8, 8, True), (3, 3, 64, 64, 64, 64, 16, True), (6, 1, 80, 48, 80, 40, 5, True), (2, 2, 16, 16, 16, 0, 4, False), (5, 5, 24, 8, 32, 24, 32, True),
+    (4, 2, 12, 20, 32, 8, 8, True), (3, 1, 10, 6, 16, 4, 8, True), (3, 3, 64, 64, 64, 64, 16, True), (6, 1, 80, 48, 80, 40, 5, True), (2, 2, 16, 16, 16, 0, 4, False), (5, 5, 24, 8, 32, 24, 32, True),
 ])
 def test_qk_norm_rope_write(src_dtype, dtype, n_q, n_kv, qk, vd, hd, rot, page_size, norm):
     """A fresh prompt, a continued portion and a decoded token in one call, from the projection itself and from partial
@@ -365,6 +389,7 @@ SINGLE_LAYERS = {
     "attention_unequal_heads_partly_rotated": single_layer(segedra.attn(3, 1, 20, 36, 0.4, window=25, rot=(3000.0, 6)), streams=None),
     "attention_window_of_a_page": single_layer(segedra.attn(2, 2, 16, 16, 1.5, window=8, rot=(10.0, 16)), streams=1),
     "attention_heads_of_a_hundred_and_twelve": single_layer(segedra.attn(2, 1, 112, 100, 0.1, window=40, rot=(500.0, 112)), streams=2),
+    "attention_sizes_that_are_no_multiple_of_four": single_layer(segedra.attn(3, 3, 10, 6, 0.4, window=9, rot=(70.0, 6), mlp=segedra.dense(21)), width=50, vocab=67, streams=3),
     "dense": single_layer(segedra.attn(1, 1, 4, 4, 0.5, window=2, rot=(10.0, 2), mlp=segedra.dense(72)), streams=4),
     "experts_all": single_layer(segedra.attn(1, 1, 4, 4, 0.5, window=2, rot=(10.0, 2), mlp=segedra.moe(12, 4, 4, 0.6, 0.5)), streams=3),
     "experts_one_of_many": single_layer(segedra.attn(1, 1, 4, 4, 0.5, window=2, rot=(10.0, 2), mlp=segedra.moe(30, 20, 1, 3.0, 4.0)), streams=None),
