@@ -35,21 +35,16 @@ extern "C" int cwm_route_tile_rows() { return TILE_ROWS; }
 // One wavefront a token: lane l holds the experts l, l + 64, ...; a choice is a vote of the lanes (the larger value, the
 // lower index among equals), so a token's router costs `top` rounds of shuffles whatever the number of experts.
 #define ROUTE_PER_LANE (ROUTE_MAX_EXPERTS / CWM_WAVE)
-__global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ chosen,
-                                                        float* __restrict__ weights, int n_tokens, int n_experts, int top, int mode,
-                                                        const float* __restrict__ correction, float scale, int renormalize) {
-  const int lane = threadIdx.x & (CWM_WAVE - 1);
-  const int t = blockIdx.x * (blockDim.x / CWM_WAVE) + threadIdx.x / CWM_WAVE;
-  if (t >= n_tokens) return;
-  const float* z = logits + (size_t)t * n_experts;
+// One token's router, by one wavefront: score[i] holds the logit of expert lane + 64 i (-inf beyond the last expert) on
+// entry; the chosen experts and their weights are written by lane 0, to chosen_out / weights_out (`top` entries each)
+// and, if given, to chosen_lds.
+__device__ __forceinline__ void route_wave(float (&score)[ROUTE_MAX_EXPERTS / CWM_WAVE], int lane, int n_experts, int top, int mode,
+                                           const float* __restrict__ correction, float scale, int renormalize,
+                                           int* __restrict__ chosen_out, float* __restrict__ weights_out, int* chosen_lds) {
   const float neg_inf = -__builtin_inff();
-  float score[ROUTE_PER_LANE], choice[ROUTE_PER_LANE];  // what a weight is made of, what an expert is chosen by
+  float choice[ROUTE_PER_LANE];  // what an expert is chosen by; score: what a weight is made of
 #pragma unroll
-  for (int i = 0; i < ROUTE_PER_LANE; ++i) {
-    const int e = lane + CWM_WAVE * i;
-    score[i] = e < n_experts ? z[e] : neg_inf;
-    choice[i] = score[i];
-  }
+  for (int i = 0; i < ROUTE_PER_LANE; ++i) choice[i] = score[i];
   if (mode == 1) {
     float largest = score[0];
 #pragma unroll
@@ -130,9 +125,26 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
 #pragma unroll
   for (int k = 0; k < ROUTE_MAX_TOP; ++k)
     if (k < top) {
-      chosen[(size_t)t * top + k] = idx[k];
-      weights[(size_t)t * top + k] = mode == 0 ? val[k] / sum : scale * (val[k] / sum);
+      chosen_out[k] = idx[k];
+      if (chosen_lds) chosen_lds[k] = idx[k];
+      weights_out[k] = mode == 0 ? val[k] / sum : scale * (val[k] / sum);
     }
+}
+
+__global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ chosen,
+                                                        float* __restrict__ weights, int n_tokens, int n_experts, int top, int mode,
+                                                        const float* __restrict__ correction, float scale, int renormalize) {
+  const int lane = threadIdx.x & (CWM_WAVE - 1);
+  const int t = blockIdx.x * (blockDim.x / CWM_WAVE) + threadIdx.x / CWM_WAVE;
+  if (t >= n_tokens) return;
+  const float* z = logits + (size_t)t * n_experts;
+  float score[ROUTE_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+    const int e = lane + CWM_WAVE * i;
+    score[i] = e < n_experts ? z[e] : -__builtin_inff();
+  }
+  route_wave(score, lane, n_experts, top, mode, correction, scale, renormalize, chosen + (size_t)t * top, weights + (size_t)t * top, nullptr);
 }
 
 extern "C" int cwm_route_top(const float* logits, int* chosen, float* weights, int n_tokens, int n_experts, int top, int mode,
@@ -148,11 +160,10 @@ extern "C" int cwm_route_top(const float* logits, int* chosen, float* weights, i
   return cwm_launch_status("route_top");
 }
 
-__global__ void __launch_bounds__(1024) group_by_expert_kernel(const int* __restrict__ chosen, int n_pairs, int n_experts,
-                                                               int* __restrict__ row_token, int* __restrict__ pair_row,
-                                                               int* __restrict__ tile_expert, int n_tiles, int top, int tile_align) {
-  __shared__ int count[ROUTE_MAX_EXPERTS];
-  __shared__ int start[ROUTE_MAX_EXPERTS];
+// The grouping, by one block; `chosen` may lie in global memory or in LDS.
+__device__ __forceinline__ void group_pairs(const int* chosen, int n_pairs, int n_experts, int* __restrict__ row_token,
+                                            int* __restrict__ pair_row, int* __restrict__ tile_expert, int n_tiles, int top,
+                                            int tile_align, int* count, int* start) {
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
   for (int i = threadIdx.x; i < n_tiles * TILE_ROWS; i += blockDim.x) row_token[i] = -1;
   for (int i = threadIdx.x; i < n_tiles; i += blockDim.x) tile_expert[i] = -1;
@@ -187,19 +198,12 @@ __global__ void __launch_bounds__(1024) group_by_expert_kernel(const int* __rest
   }
 }
 
-// tile_align: an expert's first tile lies at a multiple of so many tiles (the tiles that one block of the product takes).
-extern "C" int cwm_group_by_expert(const int* chosen, int n_tokens, int top, int n_experts, int* row_token, int* pair_row,
-                                   int* tile_expert, int n_tiles, int tile_align, hipStream_t stream) {
-  CWM_REQUIRE(chosen && row_token && pair_row && tile_expert, "group_by_expert: arguments missing");
-  CWM_REQUIRE(n_experts >= 1 && n_experts <= ROUTE_MAX_EXPERTS && top >= 1, "group_by_expert: %d experts, the kernel takes up to %d", n_experts,
-              ROUTE_MAX_EXPERTS);
-  const long n_pairs = (long)n_tokens * top;
-  CWM_REQUIRE(tile_align >= 1 && (long)n_tiles >= (n_pairs + TILE_ROWS - 1) / TILE_ROWS + (long)n_experts * tile_align,
-              "group_by_expert: %d tiles do not hold %ld pairs of %d experts", n_tiles, n_pairs, n_experts);
-  if (n_tokens <= 0) return 0;
-  hipLaunchKernelGGL(group_by_expert_kernel, dim3(1), dim3(1024), 0, stream, chosen, (int)n_pairs, n_experts, row_token, pair_row, tile_expert,
-                     n_tiles, top, tile_align);
-  return cwm_launch_status("group_by_expert");
+__global__ void __launch_bounds__(1024) group_by_expert_kernel(const int* __restrict__ chosen, int n_pairs, int n_experts,
+                                                               int* __restrict__ row_token, int* __restrict__ pair_row,
+                                                               int* __restrict__ tile_expert, int n_tiles, int top, int tile_align) {
+  __shared__ int count[ROUTE_MAX_EXPERTS];
+  __shared__ int start[ROUTE_MAX_EXPERTS];
+  group_pairs(chosen, n_pairs, n_experts, row_token, pair_row, tile_expert, n_tiles, top, tile_align, count, start);
 }
 
 // ---- the grouped product ------------------------------------------------------------------------------------- //

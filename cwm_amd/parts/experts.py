@@ -69,10 +69,7 @@ class RoutedExperts(FeedForward):
         """The same without the last kernel: every pair's row and the weights, for a consumer that adds a token's
         rows up itself (a norm that takes a `RoutedSum` as the pending result)."""
         logits = ops.linear(x, self.router, None, torch.float32)
-        if self.scores == "softmax_chosen":
-            chosen, weights = ops.route_top(logits, self.top)
-        else:
-            chosen, weights = ops.route_top(logits, self.top, self.scores, self.choice_correction, self.weight_scale, self.renormalize)
+        chosen, weights = ops.route_top(logits, self.top, self.scores, self.choice_correction, self.weight_scale, self.renormalize)
         groups = ops.group_by_expert(chosen, self.n_experts)
         if self.activation.kind == "silu":
             hidden = ops.grouped_gate_up(x, groups, self.gate, self.up)
