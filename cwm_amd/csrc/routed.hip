@@ -206,6 +206,21 @@ __global__ void __launch_bounds__(1024) group_by_expert_kernel(const int* __rest
   group_pairs(chosen, n_pairs, n_experts, row_token, pair_row, tile_expert, n_tiles, top, tile_align, count, start);
 }
 
+// tile_align: an expert's first tile lies at a multiple of so many tiles (the tiles that one block of the product takes).
+extern "C" int cwm_group_by_expert(const int* chosen, int n_tokens, int top, int n_experts, int* row_token, int* pair_row,
+                                   int* tile_expert, int n_tiles, int tile_align, hipStream_t stream) {
+  CWM_REQUIRE(chosen && row_token && pair_row && tile_expert, "group_by_expert: arguments missing");
+  CWM_REQUIRE(n_experts >= 1 && n_experts <= ROUTE_MAX_EXPERTS && top >= 1, "group_by_expert: %d experts, the kernel takes up to %d", n_experts,
+              ROUTE_MAX_EXPERTS);
+  const long n_pairs = (long)n_tokens * top;
+  CWM_REQUIRE(tile_align >= 1 && (long)n_tiles >= (n_pairs + TILE_ROWS - 1) / TILE_ROWS + (long)n_experts * tile_align,
+              "group_by_expert: %d tiles do not hold %ld pairs of %d experts", n_tiles, n_pairs, n_experts);
+  if (n_tokens <= 0) return 0;
+  hipLaunchKernelGGL(group_by_expert_kernel, dim3(1), dim3(1024), 0, stream, chosen, (int)n_pairs, n_experts, row_token, pair_row, tile_expert,
+                     n_tiles, top, tile_align);
+  return cwm_launch_status("group_by_expert");
+}
+
 // ---- the grouped product ------------------------------------------------------------------------------------- //
 // What the epilogue of a product with two weights makes of g = W0 a and u = W1 a:
 //   kind 0: silu(g) * u
