@@ -247,8 +247,9 @@ def _sink_case(dtype, n_q, n_kv, hd, page_size, lens_old, lens_new, window, seed
         k = torch.randn((n, n_kv, hd), generator=g).to(dtype)
         v = torch.randn((n, n_kv, hd), generator=g).to(dtype)
         q = torch.randn((n1, n_q, hd), generator=g).to(dtype)
-        if loud is not None and loud[0] == b:  # a key that answers the last query's head 0 loudly
-            k[loud[1], 0] = (q[-1, 0].float() * 6.0).to(dtype)
+        for lb, key_pos in ([loud] if isinstance(loud, tuple) else (loud or [])):
+            if lb == b:  # a key that answers the last query's first heads loudly (those of key/value head 0)
+                k[key_pos, 0] = (q[-1, 0].float() * 6.0).to(dtype)
         table[b, : pages_per[b]] = perm[used : used + pages_per[b]].to(torch.int32)
         used += pages_per[b]
         pos = torch.arange(n)
@@ -319,6 +320,34 @@ def test_attention_sink_where_key_ranges_are_cut_and_merged(window):
     torch.testing.assert_close(simple.double(), want, rtol=2e-2, atol=2e-2)
     without = ops.paged_attention_mfma(q, cache, table, batch, window, scale).cpu()
     assert (without.double() - want).abs().max() > 0.02
+
+
+@pytest.mark.parametrize("window,page_size", [(64, 16), (40, 8), (33, 32), (2, 16)])
+def test_attention_sink_and_a_loud_key_at_the_window_s_edges(window, page_size):
+    """The last query of a decoded token and of a prompt portion finds a loud key exactly at the window's first place
+    (it carries the row, sink or not) or one place before it (it must not be seen): a window one key off in either
+    direction changes these rows altogether.  With a window of 64 the edge lies at a page border."""
+    from cwm_amd import ops
+
+    n_q, n_kv, hd = 4, 2, 64
+    lens_old, lens_new = [300, 300, 171, 171], [1, 1, 37, 37]
+    last = [a + b - 1 for a, b in zip(lens_old, lens_new)]
+    loud = [(0, last[0] - (window - 1)), (1, last[1] - window), (2, last[2] - (window - 1)), (3, last[3] - window)]
+    for dtype in DTYPES:
+        q, cache, table, batch, sink, scale, want = _sink_case(dtype, n_q, n_kv, hd, page_size, lens_old, lens_new, window, seed=window, loud=loud)
+        # the case is sharp: had the query of sequence 1 (or 3) seen the key one place before its window, its row would be another
+        longer = _sink_case(dtype, n_q, n_kv, hd, page_size, lens_old, lens_new, window + 1, seed=window, loud=loud)[-1]
+        shorter = _sink_case(dtype, n_q, n_kv, hd, page_size, lens_old, lens_new, window - 1, seed=window, loud=loud)[-1] if window > 1 else None
+        rows = {0: 0, 1: 1, 2: 2 + 36, 3: 2 + 37 + 36}  # the last row of each sequence
+        assert (longer[rows[1]] - want[rows[1]]).abs().max() > 0.3 and (longer[rows[3]] - want[rows[3]]).abs().max() > 0.3
+        if shorter is not None:
+            assert (shorter[rows[0]] - want[rows[0]]).abs().max() > 0.3 and (shorter[rows[2]] - want[rows[2]]).abs().max() > 0.3
+        t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+        simple = ops.paged_attention_simple(q, cache, table, batch.positions, batch.seq_of_token, window, scale, sink=sink).cpu()
+        torch.testing.assert_close(simple.double(), want, **t)
+        if dtype == torch.bfloat16:
+            got = ops.paged_attention_mfma(q, cache, table, batch, window, scale, sink).cpu()
+            torch.testing.assert_close(got.double(), want, **t)
 
 
 # ---- models ------------------------------------------------------------------------------------------------------- #
